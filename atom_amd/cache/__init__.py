@@ -1,0 +1,5 @@
+from .manager import CacheManager, GroupSpec, OutOfPages, OutOfSlots, PagePool, StateSlots
+from .storage import CachePlan, CacheStorage, group_runs, plan_cache
+
+__all__ = ["CacheManager", "GroupSpec", "OutOfPages", "OutOfSlots", "PagePool", "StateSlots", "CachePlan",
+           "CacheStorage", "group_runs", "plan_cache"]

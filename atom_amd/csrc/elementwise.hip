@@ -1,0 +1,214 @@
+// Memory-bound kernels of the model step: embedding gather, RMS norm with the
+// residual sum, SiLU-gate multiply, and the fused per-head norm + rotation +
+// cache write that sits between the QKV product and attention.
+//
+// All arithmetic is in float32; activations are float32 or bfloat16 (template T),
+// the residual stream and norm weights are always float32.
+#include "common.h"
+
+// ------------------------------------------------------------------ embedding
+
+template <typename TT, typename TO>
+__global__ void embedding_kernel(const TT* __restrict__ table, const int* __restrict__ ids,
+                                 TO* __restrict__ out, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  const bool ok = id >= 0 && id < vocab;
+  const TT* row = table + (size_t)(ok ? id : 0) * hidden;
+  TO* dst = out + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    dst[i] = ok ? from_f32<TO>(to_f32(row[i])) : from_f32<TO>(0.f);
+}
+
+ATOM_EXPORT int atom_embedding(const void* table, int table_dtype, const int* ids, void* out,
+                               int out_dtype, int tokens, int hidden, int vocab, hipStream_t stream) {
+  if (tokens < 0 || hidden <= 0 || vocab <= 0) return ATOM_BAD_SHAPE;
+  if (tokens == 0) return ATOM_OK;
+  dim3 grid(tokens), block(256);
+#define LAUNCH(TT, TO) \
+  hipLaunchKernelGGL((embedding_kernel<TT, TO>), grid, block, 0, stream, (const TT*)table, ids, (TO*)out, hidden, vocab)
+  if (table_dtype == ATOM_F32 && out_dtype == ATOM_F32) LAUNCH(float, float);
+  else if (table_dtype == ATOM_BF16 && out_dtype == ATOM_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (table_dtype == ATOM_BF16 && out_dtype == ATOM_F32) LAUNCH(bf16_t, float);
+  else if (table_dtype == ATOM_F32 && out_dtype == ATOM_BF16) LAUNCH(float, bf16_t);
+  else return ATOM_BAD_DTYPE;
+#undef LAUNCH
+  return launch_status();
+}
+
+// ------------------------------------------------------------------ RMS norm
+//
+// mode 0: y = norm(x)                                   (residual untouched)
+// mode 1: residual = x (as float32); y = norm(residual)  (first layer)
+// mode 2: residual += x; y = norm(residual)
+// `rows`, when given, names the source row of each output row (x and residual are
+// read at rows[r], y is written at r) and the residual is left as it is: the sum
+// is formed only for the norm.  Used to norm just the rows whose logits are asked.
+// One block per row.
+
+template <typename T>
+__global__ void rmsnorm_kernel(const T* __restrict__ x, float* __restrict__ residual,
+                               const float* __restrict__ weight, T* __restrict__ y,
+                               const int* __restrict__ rows, int width, float eps, int mode) {
+  extern __shared__ float smem[];  // width floats + 16 for the reduction
+  float* vals = smem;
+  float* scratch = smem + width;
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  const T* xr = x + (size_t)src * width;
+  float* rr = residual ? residual + (size_t)src * width : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = to_f32(xr[i]);
+    if (mode == 2) v += rr[i];
+    vals[i] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = rsqrtf(ss / (float)width + eps);
+  T* yr = y + (size_t)r * width;
+  const bool store_residual = mode != 0 && rows == nullptr;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = vals[i];
+    if (store_residual) rr[i] = v;
+    yr[i] = from_f32<T>(v * inv * weight[i]);
+  }
+}
+
+ATOM_EXPORT int atom_rmsnorm(const void* x, void* residual, const float* weight, void* y,
+                             const int* rows, int dtype, int num_rows, int width, float eps,
+                             int mode, hipStream_t stream) {
+  if (num_rows < 0 || width <= 0 || mode < 0 || mode > 2) return ATOM_BAD_SHAPE;
+  if (mode != 0 && residual == nullptr) return ATOM_BAD_SHAPE;
+  if ((size_t)width * 4 + 64 > 64 * 1024) return ATOM_TOO_LARGE;  // the row is kept in LDS
+  if (num_rows == 0) return ATOM_OK;
+  const int threads = width >= 2048 ? 512 : (width >= 512 ? 256 : 64);
+  const size_t smem = (size_t)width * 4 + 64;
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((rmsnorm_kernel<T>), dim3(num_rows), dim3(threads), smem,
+                                                 stream, (const T*)x, (float*)residual, weight, (T*)y,
+                                                 rows, width, eps, mode));
+  return launch_status();
+}
+
+// ------------------------------------------------------------------ SiLU(gate) * up
+
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ y, int inter, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t row = idx / inter;
+  const int col = (int)(idx - row * inter);
+  const float g = to_f32(x[row * 2 * inter + col]);
+  const float u = to_f32(x[row * 2 * inter + inter + col]);
+  y[idx] = from_f32<T>(g / (1.f + expf(-g)) * u);
+}
+
+ATOM_EXPORT int atom_silu_mul(const void* x, void* y, int dtype, int rows, int inter, hipStream_t stream) {
+  if (rows < 0 || inter <= 0) return ATOM_BAD_SHAPE;
+  const size_t total = (size_t)rows * inter;
+  if (total == 0) return ATOM_OK;
+  const int threads = 256;
+  const size_t blocks = (total + threads - 1) / threads;
+  if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((silu_mul_kernel<T>), dim3((unsigned)blocks), dim3(threads), 0,
+                                                 stream, (const T*)x, (T*)y, inter, total));
+  return launch_status();
+}
+
+// ------------------------------------------------------------------ q/k norm + rotation + cache write
+//
+// Input: the QKV product [tokens, (Hq + 2 Hkv) * D], rows laid out q | k | v.
+// One wave per (token, head):
+//   q heads:  optional RMS norm over D, rotation, written to q_out [tokens, Hq, D];
+//   k heads:  optional RMS norm over D, rotation, written into the key pages;
+//   v heads:  written into the value pages as they are.
+// Rotation is NeoX style over the first `rotary_dim` elements: pairs (j, j + rotary_dim/2)
+// with cos/sin taken from float32 tables [max_pos, rotary_dim/2] at the token's position.
+// Pages: keys   [num_pages, Hkv, page_size, D]
+//        values [num_pages, Hkv, D, page_size]   (transposed: keys of a page are contiguous per d)
+// slot = page * page_size + offset; slot < 0 writes nothing (padding rows).
+// `write_kv == 0` skips k and v altogether (a layer that reads another layer's cache).
+
+template <typename T>
+__global__ void qk_norm_rope_kv_write_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const float* __restrict__ q_weight, const float* __restrict__ k_weight, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ slots,
+    int hq, int hkv, int d, int rotary_dim, int page_size, float eps, int write_kv) {
+  const int t = blockIdx.x;
+  const int head = blockIdx.y;  // 0..hq-1 q, then hkv k heads, then hkv v heads
+  const int lane = threadIdx.x;
+  const int row_width = (hq + 2 * hkv) * d;
+  const T* src = qkv + (size_t)t * row_width + (size_t)head * d;
+  const bool is_q = head < hq;
+  const bool is_k = !is_q && head < hq + hkv;
+  const int kv_head = is_q ? 0 : (is_k ? head - hq : head - hq - hkv);
+
+  int slot = -1;
+  if (!is_q) {
+    if (!write_kv) return;
+    slot = slots[t];
+    if (slot < 0) return;
+  }
+  const int page = slot / page_size;
+  const int off = slot - page * page_size;
+
+  if (!is_q && !is_k) {  // value head: plain scatter into the transposed page
+    T* dst = v_cache + ((size_t)page * hkv + kv_head) * (size_t)d * page_size + off;
+    for (int i = lane; i < d; i += kWave) dst[(size_t)i * page_size] = src[i];
+    return;
+  }
+
+  const float* weight = is_q ? q_weight : k_weight;
+  float inv = 1.f;
+  if (weight) {
+    float ss = 0.f;
+    for (int i = lane; i < d; i += kWave) {
+      const float v = to_f32(src[i]);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    inv = rsqrtf(ss / (float)d + eps);
+  }
+  T* dst = is_q ? q_out + ((size_t)t * hq + head) * d
+                : k_cache + (((size_t)page * hkv + kv_head) * page_size + off) * (size_t)d;
+  const int half = rotary_dim / 2;
+  const int pos = positions[t];
+  const float* cs = cos_table + (size_t)pos * half;
+  const float* sn = sin_table + (size_t)pos * half;
+  for (int j = lane; j < half; j += kWave) {
+    float x1 = to_f32(src[j]);
+    float x2 = to_f32(src[j + half]);
+    if (weight) {
+      x1 = x1 * inv * weight[j];
+      x2 = x2 * inv * weight[j + half];
+    }
+    const float c = cs[j], s = sn[j];
+    dst[j] = from_f32<T>(x1 * c - x2 * s);
+    dst[j + half] = from_f32<T>(x2 * c + x1 * s);
+  }
+  for (int i = rotary_dim + lane; i < d; i += kWave) {  // the part that is not rotated
+    float v = to_f32(src[i]);
+    if (weight) v = v * inv * weight[i];
+    dst[i] = from_f32<T>(v);
+  }
+}
+
+ATOM_EXPORT int atom_qk_norm_rope_kv_write(
+    const void* qkv, void* q_out, void* k_cache, void* v_cache, const float* q_weight, const float* k_weight,
+    const float* cos_table, const float* sin_table, const int* positions, const int* slots, int dtype,
+    int tokens, int hq, int hkv, int d, int rotary_dim, int page_size, float eps, int write_kv,
+    hipStream_t stream) {
+  if (tokens < 0 || hq <= 0 || hkv <= 0 || d <= 0 || page_size <= 0) return ATOM_BAD_SHAPE;
+  if (rotary_dim < 0 || rotary_dim > d || (rotary_dim & 1)) return ATOM_BAD_SHAPE;
+  if (rotary_dim > 0 && (!cos_table || !sin_table || !positions)) return ATOM_BAD_SHAPE;
+  if (write_kv && (!k_cache || !v_cache || !slots)) return ATOM_BAD_SHAPE;
+  if (hq + 2 * hkv > 65535) return ATOM_TOO_LARGE;
+  if (tokens == 0) return ATOM_OK;
+  dim3 grid(tokens, hq + 2 * hkv), block(kWave);
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<T>), grid, block, 0, stream,
+                                                 (const T*)qkv, (T*)q_out, (T*)k_cache, (T*)v_cache, q_weight,
+                                                 k_weight, cos_table, sin_table, positions, slots, hq, hkv, d,
+                                                 rotary_dim, page_size, eps, write_kv));
+  return launch_status();
+}

@@ -1,0 +1,217 @@
+"""The step function and what it stands on: the model, the cache manager, the cache's
+device memory.
+
+``EngineCore.step`` takes a batch of (request, its next tokens, the places whose logits
+are wanted): portions of prompts beside single decoded tokens, cut anywhere.  It runs
+exactly those tokens as one flat batch against the cache that earlier steps left and
+returns float32 logits at the wanted places, in the order of the entries.
+
+The reference's step (atom/model_engine/model_runner.py:3325-3415) takes either prompt
+portions or decode tokens; its batch record already lays prompt portions before decode
+tokens on one token axis (model_runner.py:441-449, scheduler.py:353-358), which is the
+layout used here for both at once.  The derived arrays are the reference's
+(atom/model_ops/attentions/backends.py:374-497): positions ``cached .. cached+n-1``,
+``slot = block_table[pos // bs] * bs + pos % bs``, ``cu_seqlens_q``, ``context_lens``,
+zero-padded block tables.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.storage import CachePlan, CacheStorage
+from ..kernels.hip import AttentionMeta
+from .context import StepContext
+
+
+@dataclass
+class StepEntry:
+    req_id: object
+    tokens: list[int]
+    want: list[int] = field(default_factory=list)   # places among ``tokens`` whose logits are wanted
+    reserve: int | None = None                      # pages are held up to this length (admission)
+
+
+class EngineCore:
+    def __init__(self, model, ops, plan: CachePlan, max_num_seqs: int, device, dtype: torch.dtype):
+        self.model = model
+        self.ops = ops
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.plan = plan
+        self.manager = CacheManager(plan.groups, max_num_seqs)
+        self.storage = CacheStorage(model, plan, max_num_seqs, self.device, dtype)
+        self.lengths: dict[object, int] = {}   # tokens of each live request that are in the cache
+        self.max_positions = model.spec.max_positions
+        self.steps_run = 0
+
+    # ------------------------------------------------------------------ requests
+
+    def is_live(self, req_id) -> bool:
+        return req_id in self.lengths
+
+    def num_cached(self, req_id) -> int:
+        return self.lengths.get(req_id, 0)
+
+    def close(self, req_id) -> None:
+        """Ends a request: its pages and state slot go back."""
+        if req_id in self.lengths:
+            del self.lengths[req_id]
+            self.manager.close(req_id)
+
+    def can_step(self, entries: list[StepEntry]) -> bool:
+        """Whether the pools hold enough free pages (and slots) for all entries at once."""
+        need = [0] * len(self.plan.groups)
+        new_requests = 0
+        for e in entries:
+            cached = self.num_cached(e.req_id)
+            if e.req_id not in self.lengths:
+                new_requests += 1
+            for gi, n in enumerate(self.manager.pages_missing(e.req_id, cached, cached + len(e.tokens), e.reserve)):
+                need[gi] += n
+        return (new_requests <= self.manager.slots.num_free
+                and all(n <= pool.num_free for n, pool in zip(need, self.manager.pools)))
+
+    # ------------------------------------------------------------------ the step
+
+    def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+        if not entries:
+            return None
+        ids = [e.req_id for e in entries]
+        if len(set(ids)) != len(ids):
+            raise ValueError("a request appears twice in one step")
+        vocab = self.model.vocab_size
+        for e in entries:
+            if not e.tokens:
+                raise ValueError(f"request {e.req_id!r}: a step entry needs at least one token")
+            if min(e.tokens) < 0 or max(e.tokens) >= vocab:
+                raise ValueError(f"request {e.req_id!r}: token id outside [0, {vocab})")
+            if any(w < 0 or w >= len(e.tokens) for w in e.want):
+                raise ValueError(f"request {e.req_id!r}: a wanted place is outside its {len(e.tokens)} tokens")
+            end = self.num_cached(e.req_id) + len(e.tokens)
+            if self.max_positions and end > self.max_positions:
+                raise ValueError(f"request {e.req_id!r}: {end} tokens exceed the model's {self.max_positions} positions")
+        if not self.can_step(entries):
+            from ..cache.manager import OutOfPages
+            raise OutOfPages("the cache cannot hold this step's tokens")
+
+        # prompt portions first, single tokens after them (stable)
+        order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) == 1)
+        fresh_slots = []
+        for e in entries:
+            if e.req_id not in self.lengths:
+                self.manager.open(e.req_id)
+                self.lengths[e.req_id] = 0
+                fresh_slots.append(self.manager.state_slot(e.req_id))
+            cached = self.lengths[e.req_id]
+            self.manager.cover(e.req_id, cached, cached + len(e.tokens), e.reserve)
+        self.storage.reset_state(fresh_slots)
+
+        ctx, token_ids, want_rows = self._build(entries, order)
+        logits = self.model.forward(ctx, token_ids, self.storage.bindings, want_rows)
+
+        for e in entries:
+            self.lengths[e.req_id] += len(e.tokens)
+            self.manager.commit(e.req_id, self.lengths[e.req_id])
+        self.steps_run += 1
+        return logits
+
+    def _build(self, entries: list[StepEntry], order: list[int]):
+        mgr = self.manager
+        num_seqs = len(entries)
+        q_lens = [len(entries[i].tokens) for i in order]
+        cached = [self.lengths[entries[i].req_id] for i in order]
+        total = sum(q_lens)
+        starts = np.zeros(num_seqs + 1, dtype=np.int32)
+        np.cumsum(q_lens, out=starts[1:])
+
+        tokens = np.empty(total, dtype=np.int32)
+        positions = np.empty(total, dtype=np.int32)
+        token_seq = np.empty(total, dtype=np.int32)
+        context_lens = np.empty(num_seqs, dtype=np.int32)
+        row_of_entry = {}
+        for b, i in enumerate(order):
+            e = entries[i]
+            s, n = int(starts[b]), q_lens[b]
+            tokens[s:s + n] = e.tokens
+            positions[s:s + n] = np.arange(cached[b], cached[b] + n, dtype=np.int32)
+            token_seq[s:s + n] = b
+            context_lens[b] = cached[b] + n
+            row_of_entry[i] = s
+        want = [row_of_entry[i] + w for i, e in enumerate(entries) for w in e.want]
+        want_rows = np.asarray(want, dtype=np.int32)
+
+        pieces = [tokens, positions, token_seq, starts, context_lens, want_rows]
+        group_shapes = []
+        for gi, g in enumerate(mgr.groups):
+            tables = [mgr.block_table(entries[i].req_id, gi) for i in order]
+            width = max(1, max(len(t) for t in tables))
+            bt = np.zeros((num_seqs, width), dtype=np.int32)
+            for b, t in enumerate(tables):
+                row = np.asarray(t, dtype=np.int32)
+                bt[b, :len(t)] = np.where(row < 0, 0, row)
+            slots = np.concatenate([mgr.slot_mapping(entries[i].req_id, gi, cached[b], q_lens[b])
+                                    for b, i in enumerate(order)]) if total else np.empty(0, np.int32)
+            pieces += [bt.reshape(-1), slots]
+            group_shapes.append(width)
+
+        # one host buffer, one copy; every array is a view of it (each padded to 4 ints)
+        offsets, cursor = [], 0
+        for p in pieces:
+            offsets.append(cursor)
+            cursor += (p.size + 3) // 4 * 4
+        host = np.zeros(max(cursor, 4), dtype=np.int32)
+        for off, p in zip(offsets, pieces):
+            host[off:off + p.size] = p
+        dev = torch.from_numpy(host).to(self.device)
+
+        def view(k):
+            return dev[offsets[k]:offsets[k] + pieces[k].size]
+
+        d_tokens, d_positions, d_token_seq, d_starts, d_ctx, d_want = (view(k) for k in range(6))
+        ctx = StepContext(ops=self.ops, dtype=self.dtype, device=self.device, num_tokens=total, num_seqs=num_seqs,
+                          positions=d_positions, seq_starts=[int(s) for s in starts[:-1]], seq_lens=q_lens,
+                          seq_cached=cached,
+                          state_slots=[mgr.state_slot(entries[i].req_id) for i in order])
+        for gi, g in enumerate(mgr.groups):
+            bt = view(6 + 2 * gi).view(num_seqs, group_shapes[gi])
+            ctx.attention[gi] = AttentionMeta(
+                token_seq=d_token_seq, positions=d_positions, block_tables=bt, cu_seqlens_q=d_starts,
+                context_lens=d_ctx, num_seqs=num_seqs, num_tokens=total, max_q_len=max(q_lens),
+                max_context_len=int(context_lens.max()), page_size=g.page_size)
+            ctx.slot_mappings[gi] = view(7 + 2 * gi)
+        return ctx, d_tokens, (d_want if want_rows.size else None)
+
+
+TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32, "bf16": torch.bfloat16, "fp32": torch.float32}
+
+
+def load_model(model_dir: str | None, *, dtype: torch.dtype, device, model_config=None, source=None, progress=None):
+    """Builds the model that ``config.json`` names through the registry and fills its
+    weights from the folder's safetensors (or from ``source``, e.g. random weights)."""
+    from ..config.model_config import read_config_json
+    from ..config.registry import build_model, model_config_from_dict
+    from ..weights.loader import SafetensorsFolder, load_weights
+
+    if model_config is None:
+        model_config = model_config_from_dict(read_config_json(model_dir))
+    model = build_model(model_config)
+    if source is None:
+        source = SafetensorsFolder(model_dir)
+    load_weights(model, source, device, dtype, progress)
+    return model, model_config
+
+
+def build_core(model, ops, *, dtype: torch.dtype, device, page_size: int = 16, num_pages: int | None = None,
+               budget_bytes: int | None = None, max_num_seqs: int = 4, max_model_len: int = 0,
+               max_num_batched_tokens: int = 0) -> EngineCore:
+    from ..cache.storage import plan_cache
+
+    plan = plan_cache(model, page_size, dtype, num_pages=num_pages, budget_bytes=budget_bytes,
+                      max_num_seqs=max_num_seqs, max_model_len=max_model_len,
+                      max_num_batched_tokens=max_num_batched_tokens)
+    return EngineCore(model, ops, plan, max_num_seqs, device, dtype)

@@ -1,0 +1,266 @@
+"""The engine's kernel library: hand-written HIP for gfx950 behind a C interface,
+called through ctypes on PyTorch's current stream.
+
+Every method checks on the host that the operands have the shapes, types and
+device the kernel and its grid assume, and raises before anything is launched.
+There is no fallback: without a GPU or without the built library, construction fails.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+
+import torch
+
+from . import build as _build
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+_STATUS = {
+    1: "unsupported element type",
+    2: "operand shapes do not fit the kernel",
+    3: "unsupported configuration",
+    4: "kernel launch failed",
+    5: "a size exceeds what the kernel can hold",
+}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+@dataclass
+class AttentionMeta:
+    """What attention needs to know about a step's batch, on the device, for one
+    group of layers that share block tables.
+
+    token_seq[t]      index of the request (row of block_tables) token t belongs to, -1 for padding
+    positions[t]      absolute position of token t in its request
+    block_tables      [num_seqs, max_blocks] page ids of each request, in order of position
+    cu_seqlens_q      [num_seqs + 1] first token of each request in the flat token axis
+    context_lens      [num_seqs] keys of each request once this step's tokens are written
+    The three ``max_``/``num_`` numbers are host copies used to pick a kernel and its grid.
+    """
+
+    token_seq: torch.Tensor
+    positions: torch.Tensor
+    block_tables: torch.Tensor
+    cu_seqlens_q: torch.Tensor
+    context_lens: torch.Tensor
+    num_seqs: int
+    num_tokens: int
+    max_q_len: int
+    max_context_len: int
+    page_size: int
+
+
+def _ptr(t: torch.Tensor | None):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+class HipKernels:
+    """Loads (building first if need be) the kernel library and binds its entry points."""
+
+    name = "hip"
+
+    def __init__(self, device: str | torch.device = "cuda:0"):
+        if not torch.cuda.is_available():
+            raise KernelError(
+                "atom_amd runs on an AMD GPU only: torch.cuda.is_available() is False and there is no CPU path")
+        self.device = torch.device(device)
+        path = _build.build()
+        try:
+            self.lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError(f"could not load the kernel library {path}: {e}") from e
+        self.path = path
+        for fn in ("atom_embedding", "atom_rmsnorm", "atom_silu_mul", "atom_qk_norm_rope_kv_write",
+                   "atom_paged_attention_generic", "atom_gemm_f32", "atom_sample", "atom_exponential_noise"):
+            getattr(self.lib, fn).restype = ctypes.c_int
+        self.allow_library_gemm = True
+
+    # ------------------------------------------------------------------ helpers
+
+    def _stream(self):
+        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _check(self, name: str, t: torch.Tensor, dtype=None, shape=None):
+        if not isinstance(t, torch.Tensor):
+            raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
+        if t.device.type != "cuda":
+            raise KernelError(f"{name}: must live on the GPU, is on {t.device}")
+        if not t.is_contiguous():
+            raise KernelError(f"{name}: must be contiguous (shape {tuple(t.shape)}, strides {t.stride()})")
+        if dtype is not None:
+            allowed = dtype if isinstance(dtype, (tuple, list)) else (dtype,)
+            if t.dtype not in allowed:
+                raise KernelError(f"{name}: element type {t.dtype} not in {allowed}")
+        if shape is not None:
+            if len(shape) != t.dim() or any(s is not None and s != a for s, a in zip(shape, t.shape)):
+                raise KernelError(f"{name}: shape {tuple(t.shape)} does not match {tuple(shape)}")
+        return t
+
+    def _done(self, what: str, status: int):
+        if status != 0:
+            raise KernelError(f"{what}: {_STATUS.get(status, f'status {status}')}")
+
+    @staticmethod
+    def _code(t: torch.Tensor) -> int:
+        try:
+            return _DTYPE_CODE[t.dtype]
+        except KeyError:
+            raise KernelError(f"element type {t.dtype} is not supported (float32 and bfloat16 are)") from None
+
+    # ------------------------------------------------------------------ kernels
+
+    def embedding(self, table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        vocab, hidden = table.shape
+        tokens = ids.numel()
+        self._check("embedding table", table, (torch.float32, torch.bfloat16))
+        self._check("token ids", ids, torch.int32, (tokens,))
+        self._check("embedding out", out, (torch.float32, torch.bfloat16), (tokens, hidden))
+        self._done("embedding", self.lib.atom_embedding(
+            _ptr(table), self._code(table), _ptr(ids), _ptr(out), self._code(out), tokens, hidden, vocab,
+            self._stream()))
+        return out
+
+    def rmsnorm(self, x, weight, eps: float, out, residual=None, mode: str = "plain", rows=None):
+        """mode 'plain': out = norm(x); 'init': residual = x, out = norm(x);
+        'add': residual += x, out = norm(residual).  With ``rows`` only those source
+        rows are normed (into out[0..len(rows))) and the residual is not written."""
+        width = x.shape[-1]
+        code = {"plain": 0, "init": 1, "add": 2}[mode]
+        self._check("norm input", x, (torch.float32, torch.bfloat16), (None, width))
+        self._check("norm weight", weight, torch.float32, (width,))
+        n_out = rows.numel() if rows is not None else x.shape[0]
+        self._check("norm out", out, x.dtype, (n_out, width))
+        if code:
+            if residual is None:
+                raise KernelError("norm: this mode needs the residual stream")
+            self._check("residual", residual, torch.float32, tuple(x.shape))
+        if rows is not None:
+            self._check("norm rows", rows, torch.int32, (n_out,))
+        self._done("rmsnorm", self.lib.atom_rmsnorm(
+            _ptr(x), _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows), self._code(x), n_out, width,
+            ctypes.c_float(eps), code, self._stream()))
+        return out
+
+    def silu_mul(self, x, out):
+        rows, two = x.shape
+        if two % 2:
+            raise KernelError("silu_mul: the input width must be even (gate | up)")
+        self._check("silu_mul input", x, (torch.float32, torch.bfloat16))
+        self._check("silu_mul out", out, x.dtype, (rows, two // 2))
+        self._done("silu_mul", self.lib.atom_silu_mul(_ptr(x), _ptr(out), self._code(x), rows, two // 2,
+                                                      self._stream()))
+        return out
+
+    def qk_norm_rope_kv_write(self, qkv, q_out, k_cache, v_cache, q_weight, k_weight, cos, sin, positions,
+                              slots, num_heads: int, num_kv_heads: int, head_dim: int, rotary_dim: int,
+                              page_size: int, eps: float, write_kv: bool = True):
+        tokens = qkv.shape[0]
+        dt = qkv.dtype
+        self._check("qkv", qkv, (torch.float32, torch.bfloat16), (tokens, (num_heads + 2 * num_kv_heads) * head_dim))
+        self._check("q out", q_out, dt, (tokens, num_heads, head_dim))
+        if write_kv:
+            self._check("key pages", k_cache, dt, (None, num_kv_heads, page_size, head_dim))
+            self._check("value pages", v_cache, dt, (k_cache.shape[0], num_kv_heads, head_dim, page_size))
+            self._check("slot mapping", slots, torch.int32, (tokens,))
+        for name, w in (("q norm weight", q_weight), ("k norm weight", k_weight)):
+            if w is not None:
+                self._check(name, w, torch.float32, (head_dim,))
+        if rotary_dim:
+            self._check("cos table", cos, torch.float32, (None, rotary_dim // 2))
+            self._check("sin table", sin, torch.float32, tuple(cos.shape))
+            self._check("positions", positions, torch.int32, (tokens,))
+        self._done("qk_norm_rope_kv_write", self.lib.atom_qk_norm_rope_kv_write(
+            _ptr(qkv), _ptr(q_out), _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None,
+            _ptr(q_weight), _ptr(k_weight), _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None,
+            _ptr(positions) if rotary_dim else None, _ptr(slots) if write_kv else None, self._code(qkv), tokens,
+            num_heads, num_kv_heads, head_dim, rotary_dim, page_size, ctypes.c_float(eps), int(bool(write_kv)),
+            self._stream()))
+        return q_out
+
+    def paged_attention(self, q, k_cache, v_cache, out, meta: AttentionMeta, scale: float,
+                        window: int | None = None):
+        tokens, hq, d = q.shape
+        _, hkv, page_size, _ = k_cache.shape
+        dt = q.dtype
+        if hq % hkv:
+            raise KernelError(f"attention: {hq} query heads are not a multiple of {hkv} key/value heads")
+        self._check("q", q, (torch.float32, torch.bfloat16))
+        self._check("key pages", k_cache, dt, (None, hkv, page_size, d))
+        self._check("value pages", v_cache, dt, (k_cache.shape[0], hkv, d, page_size))
+        self._check("attention out", out, dt, (tokens, hq, d))
+        self._check("token_seq", meta.token_seq, torch.int32, (tokens,))
+        self._check("positions", meta.positions, torch.int32, (tokens,))
+        self._check("block tables", meta.block_tables, torch.int32, (None, None))
+        if meta.page_size != page_size:
+            raise KernelError("attention: the batch's page size differs from the cache's")
+        if meta.max_context_len > meta.block_tables.shape[1] * page_size:
+            raise KernelError("attention: a context is longer than its block table can name")
+        self._done("paged_attention", self.lib.atom_paged_attention_generic(
+            _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.token_seq), _ptr(meta.positions),
+            _ptr(meta.block_tables), meta.block_tables.shape[1], self._code(q), tokens, hq, hkv, d, page_size,
+            ctypes.c_float(scale), int(window or 0), self._stream()))
+        return out
+
+    def linear(self, x, weight, bias=None, out_dtype=None):
+        """``x @ weight.T (+ bias)``.  bfloat16 operands go to the BLAS library, as the
+        reference's engine does for its matrix products; anything with a float32 operand
+        runs this library's own float32 kernel (plain FMA, no reduced-precision mode)."""
+        m, k = x.shape
+        n = weight.shape[0]
+        self._check("linear input", x, (torch.float32, torch.bfloat16))
+        self._check("linear weight", weight, (torch.float32, torch.bfloat16), (n, k))
+        out_dtype = out_dtype or x.dtype
+        if bias is not None:
+            self._check("linear bias", bias, torch.float32, (n,))
+        if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and self.allow_library_gemm:
+            y = torch.nn.functional.linear(x, weight)
+            if bias is not None:
+                y = (y.float() + bias)
+            return y.to(out_dtype)
+        y = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        self._done("gemm_f32", self.lib.atom_gemm_f32(
+            _ptr(x), self._code(x), _ptr(weight), self._code(weight), _ptr(bias), _ptr(y), self._code(y), m, n, k,
+            self._stream()))
+        return y
+
+    def sample(self, logits, temperatures, out, top_ks=None, top_ps=None, noise=None, seeds=None, counters=None,
+               eps: float = 1e-10):
+        rows, vocab = logits.shape
+        self._check("logits", logits, torch.float32)
+        self._check("sampled ids", out, torch.int32, (rows,))
+        if temperatures is not None:
+            self._check("temperatures", temperatures, torch.float32, (rows,))
+        if top_ks is not None:
+            self._check("top_ks", top_ks, torch.int32, (rows,))
+        if top_ps is not None:
+            self._check("top_ps", top_ps, torch.float32, (rows,))
+        stride = 0
+        if noise is not None:
+            self._check("noise", noise, torch.float32, (None, vocab))
+            if noise.shape[0] not in (1, rows):
+                raise KernelError("noise must have one row or one per logits row")
+            stride = vocab if noise.shape[0] == rows and rows > 1 else 0
+        else:
+            if temperatures is not None and (seeds is None or counters is None):
+                raise KernelError("sampling without given noise needs seeds and counters")
+        if seeds is not None:
+            self._check("seeds", seeds, torch.int64, (rows,))
+            self._check("counters", counters, torch.int64, (rows,))
+        self._done("sample", self.lib.atom_sample(
+            _ptr(logits), _ptr(temperatures), _ptr(top_ks), _ptr(top_ps), _ptr(noise), ctypes.c_long(stride),
+            _ptr(seeds), _ptr(counters), _ptr(out), rows, vocab, ctypes.c_float(eps), self._stream()))
+        return out
+
+    def exponential_noise(self, seeds, counters, vocab: int):
+        rows = seeds.numel()
+        self._check("seeds", seeds, torch.int64, (rows,))
+        self._check("counters", counters, torch.int64, (rows,))
+        out = torch.empty((rows, vocab), dtype=torch.float32, device=seeds.device)
+        self._done("exponential_noise", self.lib.atom_exponential_noise(
+            _ptr(out), _ptr(seeds), _ptr(counters), rows, vocab, self._stream()))
+        return out

@@ -1,0 +1,86 @@
+"""Grouped-query attention over the paged cache.
+
+The order of operations is atom/models/qwen3.py:146-162: one packed QKV product
+(rows q | k | v, atom/model_ops/linear.py:1835-1848), RMS norm of every q and k
+head over the head dimension (optional), rotation, the new keys and values written
+to their pages, attention of the new queries over the pages, output projection.
+Norm, rotation and the cache write are one kernel; the scale defaults to
+``head_dim ** -0.5`` (qwen3.py:88).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .base import MIXERS, POSITION_ENCODINGS, KVCacheNeed, Mixer, ParamSpec, PartChoice
+
+
+class GroupedQueryAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 qkv_bias: bool = False, out_bias: bool = False, qk_norm: bool = False, norm_eps: float = 1e-6,
+                 scale: float | None = None, window: int | None = None,
+                 position_encoding: PartChoice | None = None, prefix: str = "",
+                 names: dict[str, str] | None = None):
+        super().__init__(prefix)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.qkv_bias = qkv_bias
+        self.out_bias = out_bias
+        self.qk_norm = qk_norm
+        self.norm_eps = float(norm_eps)
+        self.scale = float(scale) if scale is not None else head_dim ** -0.5
+        self.window = window
+        self.names = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "q_norm": "q_norm",
+                      "k_norm": "k_norm", **(names or {})}
+        self.rope = position_encoding.build(POSITION_ENCODINGS, head_dim=head_dim) if position_encoding else None
+
+    def children(self):
+        return [self.rope] if self.rope is not None else []
+
+    def cache_need(self):
+        return KVCacheNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    def param_specs(self):
+        n = self.names
+        q_rows, kv_rows = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
+        specs = {
+            "qkv.weight": ParamSpec.stacked(
+                [(f"{n['q']}.weight", q_rows), (f"{n['k']}.weight", kv_rows), (f"{n['v']}.weight", kv_rows)],
+                (self.hidden_size,)),
+            "o.weight": ParamSpec.single(f"{n['o']}.weight", (self.hidden_size, q_rows)),
+        }
+        if self.qkv_bias:
+            specs["qkv.bias"] = ParamSpec.stacked(
+                [(f"{n['q']}.bias", q_rows), (f"{n['k']}.bias", kv_rows), (f"{n['v']}.bias", kv_rows)], (),
+                kind="vector")
+        if self.out_bias:
+            specs["o.bias"] = ParamSpec.single(f"{n['o']}.bias", (self.hidden_size,), kind="vector")
+        if self.qk_norm:
+            specs["q_norm.weight"] = ParamSpec.single(f"{n['q_norm']}.weight", (self.head_dim,), kind="vector",
+                                                      init="one_plus_normal")
+            specs["k_norm.weight"] = ParamSpec.single(f"{n['k_norm']}.weight", (self.head_dim,), kind="vector",
+                                                      init="one_plus_normal")
+        return specs
+
+    def forward(self, ctx, x, cache):
+        ops = ctx.ops
+        tokens = x.shape[0]
+        qkv = ops.linear(x, self.params["qkv.weight"], self.p("qkv.bias"))
+        q = torch.empty((tokens, self.num_heads, self.head_dim), dtype=x.dtype, device=x.device)
+        meta = ctx.attention[cache.group]
+        rope = self.rope
+        ops.qk_norm_rope_kv_write(
+            qkv, q, cache.k_cache, cache.v_cache, self.p("q_norm.weight"), self.p("k_norm.weight"),
+            rope.cos if rope else None, rope.sin if rope else None, ctx.positions,
+            ctx.slot_mappings[cache.group], self.num_heads, self.num_kv_heads, self.head_dim,
+            rope.rotary_dim if rope else 0, meta.page_size, self.norm_eps, write_kv=cache.writes)
+        out = torch.empty_like(q)
+        ops.paged_attention(q, cache.k_cache, cache.v_cache, out, meta, self.scale, self.window)
+        return ops.linear(out.view(tokens, self.num_heads * self.head_dim), self.params["o.weight"], self.p("o.bias"))
+
+
+MIXERS.register("attention", GroupedQueryAttention)
