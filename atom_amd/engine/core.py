@@ -48,6 +48,7 @@ class EngineCore:
         self.lengths: dict[object, int] = {}   # tokens of each live request that are in the cache
         self.max_positions = model.spec.max_positions
         self.steps_run = 0
+        self._fresh_slots: list[int] = []      # slots claimed since the last step: zeroed before it runs
 
     # ------------------------------------------------------------------ requests
 
@@ -56,6 +57,15 @@ class EngineCore:
 
     def num_cached(self, req_id) -> int:
         return self.lengths.get(req_id, 0)
+
+    def open(self, req_id) -> None:
+        """Registers a request: it holds a state slot from now to ``close``.  A step opens
+        unknown requests itself; a scheduler opens them when it admits them, to take pages."""
+        if req_id in self.lengths:
+            return
+        self.manager.open(req_id)
+        self.lengths[req_id] = 0
+        self._fresh_slots.append(self.manager.state_slot(req_id))
 
     def close(self, req_id) -> None:
         """Ends a request: its pages and state slot go back."""
@@ -101,15 +111,12 @@ class EngineCore:
 
         # prompt portions first, single tokens after them (stable)
         order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) == 1)
-        fresh_slots = []
         for e in entries:
-            if e.req_id not in self.lengths:
-                self.manager.open(e.req_id)
-                self.lengths[e.req_id] = 0
-                fresh_slots.append(self.manager.state_slot(e.req_id))
+            self.open(e.req_id)
             cached = self.lengths[e.req_id]
             self.manager.cover(e.req_id, cached, cached + len(e.tokens), e.reserve)
-        self.storage.reset_state(fresh_slots)
+        self.storage.reset_state(self._fresh_slots)
+        self._fresh_slots = []
 
         ctx, token_ids, want_rows = self._build(entries, order)
         logits = self.model.forward(ctx, token_ids, self.storage.bindings, want_rows)

@@ -1,0 +1,189 @@
+"""The Python entry point, in ATOM's manner (atom/model_engine/llm_engine.py:36-260):
+
+    llm = LLMEngine(model_dir, **config_kwargs)
+    outputs = llm.generate(prompts, sampling_params)   # prompts: strings or token-id lists
+
+Each output is a dict with the reference's keys (llm_engine.py:752-762): ``text``,
+``token_ids``, ``logprobs``, ``latency``, ``finish_reason``, ``num_tokens_input``,
+``num_tokens_output``, ``ttft``, ``tpot``.  Everything runs in this process: one step is
+schedule -> step function -> sampler -> postprocess.
+"""
+
+from __future__ import annotations
+
+import logging
+import os
+import time
+
+import torch
+
+from ..config.engine_config import Config
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+from .core import TORCH_DTYPES, build_core, load_model
+from .scheduler import Scheduler
+from .sequence import Sequence
+
+logger = logging.getLogger("atom_amd")
+
+
+def _load_tokenizer(path: str):
+    """A tokenizer if the folder has one (atom/model_engine/llm_engine.py:23-33); prompts
+    given as token ids need none."""
+    if not any(os.path.isfile(os.path.join(path, f)) for f in ("tokenizer.json", "tokenizer.model", "vocab.json")):
+        return None
+    from transformers import AutoTokenizer
+
+    return AutoTokenizer.from_pretrained(path)
+
+
+class LLMEngine:
+    def __init__(self, model: str, tokenizer=None, ops=None, weight_source=None, **kwargs):
+        kwargs = {k: v for k, v in kwargs.items() if k in Config.__dataclass_fields__}
+        self.config = cfg = Config(model, **kwargs)
+        if cfg.enable_prefix_caching:
+            logger.warning("prefix caching is not built in this engine; running without it")
+        self.tokenizer = tokenizer if tokenizer is not None else (
+            _load_tokenizer(model) if isinstance(model, str) and os.path.isdir(model) else None)
+        self.dtype = TORCH_DTYPES[cfg.dtype]
+        if ops is None:
+            from ..kernels.hip import HipKernels
+
+            ops = HipKernels(cfg.device)
+        self.ops = ops
+        source = weight_source
+        if source is None and cfg.load_dummy:
+            from ..config.registry import build_model
+            from ..weights.random_init import RandomSource
+
+            source = RandomSource(build_model(cfg.model_config), cfg.seed)
+        self.model, _ = load_model(cfg.model, dtype=self.dtype, device=cfg.device, model_config=cfg.model_config,
+                                   source=source)
+        self.core = build_core(
+            self.model, ops, dtype=self.dtype, device=cfg.device, page_size=cfg.kv_cache_block_size,
+            num_pages=cfg.num_kvcache_blocks if cfg.num_kvcache_blocks > 0 else None,
+            budget_bytes=self._cache_budget() if cfg.num_kvcache_blocks <= 0 else None,
+            max_num_seqs=cfg.max_num_seqs, max_model_len=cfg.max_model_len,
+            max_num_batched_tokens=cfg.max_num_batched_tokens)
+        self.scheduler = Scheduler(cfg, self.core)
+        self.sampler = Sampler(ops, cfg.device)
+        self.seqs: dict[int, Sequence] = {}
+        self._profiler = None
+
+    def _cache_budget(self) -> int:
+        """Bytes for the cache: the share of device memory ``gpu_memory_utilization`` allows
+        minus what is in use, with a 2 % margin (atom/model_engine/model_runner.py:1591-1611)."""
+        dev = torch.device(self.config.device)
+        if dev.type != "cuda":
+            return 64 << 20
+        free, total = torch.cuda.mem_get_info(dev)
+        used = total - free
+        budget = int(total * self.config.gpu_memory_utilization) - used - int(total * 0.02)
+        return max(0, min(budget, free))
+
+    # ------------------------------------------------------------------ requests
+
+    def add_request(self, prompt, sampling_params: SamplingParams | None = None) -> list[Sequence]:
+        sp = sampling_params or SamplingParams()
+        if isinstance(prompt, str):
+            if self.tokenizer is None:
+                raise ValueError("a text prompt needs a tokenizer; this model folder has none (pass token ids)")
+            token_ids = self.tokenizer.encode(prompt)
+        else:
+            token_ids = [int(t) for t in prompt]
+        if not token_ids:
+            raise ValueError("an empty prompt cannot be run")
+        stop_seqs = []
+        if sp.stop_strings:   # atom/model_engine/llm_engine.py:661-671
+            if self.tokenizer is None:
+                raise ValueError("stop_strings need a tokenizer")
+            stop_seqs = [self.tokenizer.encode(s, add_special_tokens=False) for s in sp.stop_strings]
+        out = []
+        for k in range(sp.n):
+            base = sp.seed if sp.seed is not None else self.config.seed
+            seq = Sequence(token_ids, sp, stop_seqs)
+            seq.seed = (base * 1_000_003 + seq.id * 7919 + k) if sp.seed is None else (base + k)
+            self.seqs[seq.id] = seq
+            self.scheduler.add(seq)
+            out.append(seq)
+        return out
+
+    def is_finished(self) -> bool:
+        return self.scheduler.is_finished()
+
+    # ------------------------------------------------------------------ one step
+
+    def step(self) -> list[Sequence]:
+        """Runs one scheduled batch; returns the sequences that left in it."""
+        batch = self.scheduler.schedule()
+        done = self.scheduler.take_rejected()
+        if batch is None:
+            return done
+        start = time.time()
+        logits = self.core.step(batch.entries())
+        sampled = {}
+        finals = [it for it in batch.items if it.is_final]
+        if finals:
+            tokens = self.sampler(logits, [it.seq.sampling_params for it in finals],
+                                  [it.seq.seed for it in finals],
+                                  [it.seq.num_completion_tokens for it in finals])
+            want_lp = any(it.seq.sampling_params.logprobs for it in finals)
+            lps = self.sampler.logprobs(logits, tokens).tolist() if want_lp else None
+            host = tokens.tolist()
+            for k, it in enumerate(finals):
+                sampled[it.seq.id] = host[k]
+                if lps is not None and it.seq.sampling_params.logprobs:
+                    it.seq.logprobs.append(lps[k])
+        done += self.scheduler.postprocess(batch, sampled, time.time() - start)
+        return done
+
+    # ------------------------------------------------------------------ generate
+
+    def _output(self, seq: Sequence) -> dict:
+        ids = seq.completion_token_ids
+        text = self.tokenizer.decode(ids) if self.tokenizer is not None else ""
+        n = seq.num_completion_tokens
+        ttft = seq.first_token_time - seq.arrive_time if seq.first_token_time else 0.0
+        tpot = (seq.leave_time - seq.first_token_time) / (n - 1) if n > 1 else 0.0
+        return {"text": text, "token_ids": ids, "logprobs": seq.logprobs or None,
+                "latency": seq.leave_time - seq.arrive_time, "finish_reason": seq.leave_reason,
+                "num_tokens_input": seq.num_prompt_tokens, "num_tokens_output": n, "ttft": ttft, "tpot": tpot}
+
+    def generate(self, prompts, sampling_params: SamplingParams | list[SamplingParams] | None = None) -> list[dict]:
+        if not isinstance(sampling_params, list):
+            sampling_params = [sampling_params or SamplingParams()] * len(prompts)
+        if len(sampling_params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt, or one for all")
+        pending = {}
+        for prompt, sp in zip(prompts, sampling_params):
+            for seq in self.add_request(prompt, sp):
+                pending[seq.id] = seq
+        outputs = {}
+        while pending:
+            for seq in self.step():
+                if seq.id in pending:
+                    outputs[seq.id] = self._output(seq)
+                    del pending[seq.id]
+                    self.seqs.pop(seq.id, None)
+            if self.scheduler.is_finished() and pending:
+                raise RuntimeError(f"the scheduler is idle but {len(pending)} request(s) never finished")
+        return [outputs[i] for i in sorted(outputs)]
+
+    # ------------------------------------------------------------------ profiling
+
+    def start_profile(self):
+        """torch.profiler trace into ``torch_profiler_dir`` (atom/model_engine/model_runner.py:1025-1129)."""
+        if not self.config.torch_profiler_dir or self._profiler is not None:
+            return
+        from torch.profiler import ProfilerActivity, profile
+
+        self._profiler = profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA])
+        self._profiler.__enter__()
+
+    def stop_profile(self):
+        if self._profiler is None:
+            return
+        self._profiler.__exit__(None, None, None)
+        os.makedirs(self.config.torch_profiler_dir, exist_ok=True)
+        self._profiler.export_chrome_trace(os.path.join(self.config.torch_profiler_dir, "trace.json"))
+        self._profiler = None

@@ -1,0 +1,307 @@
+"""Continuous batching above the step function.
+
+Rules kept from the reference's scheduler (atom/model_engine/scheduler.py): FIFO
+admission with head-of-line blocking (:1187-1347), ``max_num_seqs`` and a per-step token
+budget ``max_num_batched_tokens`` (:1180-1186), prompts cut into portions under the
+budget with a truncated portion floored to a multiple of ``max(block_size, 64)`` and a
+sliver not scheduled unless the batch is empty (:1733-1753), permanent rejection of
+requests that can never run (:989-1050), preemption of the last running request when
+pages run out, the preempted request going back to the head of the waiting queue and
+later prefilling prompt plus generated tokens (:1917-1952, :1277-1283), and the finishing
+rules in their order (:2296-2329).
+
+What differs: the reference schedules prompt portions *or* decode tokens per step
+(:1370-1429); here one step holds both.  Running requests that decode are scheduled
+first (one token each), then unfinished prompts, then new admissions, all under the one
+token budget.  Pages are taken when a request is scheduled: a group that keeps every key
+reserves the whole prompt at admission (as ``BlockManager.allocate`` does, block_manager.py
+:447-470), a window group only what the step needs.
+"""
+
+from __future__ import annotations
+
+import time
+from collections import deque
+from dataclasses import dataclass, field
+
+from .core import StepEntry
+from .sequence import Sequence, SequenceStatus
+
+
+@dataclass
+class ScheduledItem:
+    seq: Sequence
+    num_tokens: int          # tokens of this step
+    start: int               # = seq.num_cached_tokens when scheduled
+    is_decode: bool
+    is_final: bool           # after this step the sequence has all its tokens in the cache
+
+
+@dataclass
+class ScheduledBatch:
+    items: list[ScheduledItem] = field(default_factory=list)
+
+    @property
+    def total_tokens(self) -> int:
+        return sum(i.num_tokens for i in self.items)
+
+    @property
+    def num_decode(self) -> int:
+        return sum(1 for i in self.items if i.is_decode)
+
+    @property
+    def num_prefill(self) -> int:
+        return sum(1 for i in self.items if not i.is_decode)
+
+    def entries(self) -> list[StepEntry]:
+        out = []
+        for it in self.items:
+            tokens = it.seq.token_ids[it.start:it.start + it.num_tokens]
+            want = [it.num_tokens - 1] if it.is_final else []
+            reserve = it.seq.num_tokens if not it.is_decode else None
+            out.append(StepEntry(it.seq.id, tokens, want, reserve))
+        return out
+
+
+class Scheduler:
+    def __init__(self, config, core):
+        """``core`` is the ``EngineCore`` whose cache manager this scheduler takes pages from."""
+        self.core = core
+        self.manager = core.manager
+        self.max_num_seqs = config.max_num_seqs
+        self.max_num_batched_tokens = config.max_num_batched_tokens
+        self.max_model_len = config.max_model_len
+        self.block_size = config.kv_cache_block_size
+        self.enable_chunked_prefill = config.enable_chunked_prefill
+        self.long_prefill_token_threshold = config.long_prefill_token_threshold
+        self.delay_factor = config.scheduler_delay_factor
+        self.eos_token_id = config.eos_token_id
+        self.stop_token_ids = set(config.stop_token_ids or [])
+        self.waiting: deque[Sequence] = deque()
+        self.running: deque[Sequence] = deque()
+        self._rejected: list[Sequence] = []
+        self.total_preemptions = 0
+        self._last_prompt_time = 0.0
+        self._last_prompt_latency = 0.0
+
+    # ------------------------------------------------------------------ queues
+
+    def add(self, seq: Sequence) -> None:
+        self.waiting.append(seq)
+
+    def extend(self, seqs) -> None:
+        for s in seqs:
+            self.add(s)
+
+    def is_finished(self) -> bool:
+        return not self.waiting and not self.running and not self._rejected
+
+    def take_rejected(self) -> list[Sequence]:
+        out, self._rejected = self._rejected, []
+        return out
+
+    # ------------------------------------------------------------------ helpers
+
+    def _unschedulable_reason(self, seq: Sequence) -> str | None:
+        """Why a request can never run, or None (atom/model_engine/scheduler.py:989-1050)."""
+        n = seq.num_tokens
+        if n > self.max_model_len:
+            return f"{n} tokens exceed max_model_len {self.max_model_len}"
+        if not self.enable_chunked_prefill and n > self.max_num_batched_tokens:
+            return f"{n} tokens exceed max_num_batched_tokens {self.max_num_batched_tokens} with chunked prefill off"
+        for gi, g in enumerate(self.manager.groups):
+            if g.window is None:
+                need = -(-n // g.page_size)
+                if need > g.num_pages:
+                    return f"needs {need} cache pages, the pool has {g.num_pages}"
+        return None
+
+    def _chunked_prefill_size(self, num_new: int, budget_left: int, batched: int) -> int:
+        """Tokens to run this step or 0 to wait (atom/model_engine/scheduler.py:1733-1753)."""
+        chunk = min(num_new, budget_left)
+        if chunk >= num_new:
+            return chunk
+        aligned = chunk - chunk % max(self.block_size, 64)
+        return aligned or (0 if batched else chunk)
+
+    def _prefill_chunk_for_budget(self, num_new: int, budget_left: int, batched: int) -> int | None:
+        """atom/model_engine/scheduler.py:1755-1767."""
+        if self.enable_chunked_prefill:
+            return self._chunked_prefill_size(num_new, budget_left, batched) or None
+        if num_new > budget_left and batched > 0:
+            return None
+        return num_new
+
+    def _passed_delay(self, now: float) -> bool:
+        """atom/model_engine/scheduler.py:2761-2777: hold new prompts until the oldest waiting
+        request has waited ``delay_factor`` times the last prompt step's latency."""
+        if self.delay_factor <= 0 or not self.waiting or not self.running:
+            return True
+        earliest = min(s.arrive_time for s in self.waiting)
+        return (now - earliest) > self.delay_factor * self._last_prompt_latency
+
+    def preempt(self, seq: Sequence) -> None:
+        """atom/model_engine/scheduler.py:1928-1952: back to the head of the waiting queue, pages
+        and slot given back; on re-admission prompt plus generated tokens are prefilled."""
+        self.total_preemptions += 1
+        seq.num_preemptions += 1
+        seq.status = SequenceStatus.WAITING
+        seq.is_partial_prefill = False
+        seq.num_cached_tokens = 0
+        self.core.close(seq.id)
+        self.waiting.appendleft(seq)
+
+    def _preempt_one_running(self, protect: set[int]) -> bool:
+        """Preempts the last running request that is not scheduled in this step."""
+        for index in range(len(self.running) - 1, -1, -1):
+            cand = self.running[index]
+            if cand.id in protect:
+                continue
+            del self.running[index]
+            self.preempt(cand)
+            return True
+        return False
+
+    # ------------------------------------------------------------------ schedule
+
+    def schedule(self) -> ScheduledBatch | None:
+        if not self.running and not self.waiting:
+            return None
+        batch = ScheduledBatch()
+        scheduled: set[int] = set()
+        batched = 0
+        mgr = self.manager
+
+        # ---- running requests that decode: one token each
+        for seq in list(self.running):
+            if seq.status != SequenceStatus.RUNNING or seq.is_partial_prefill or seq.id in scheduled:
+                continue
+            if seq not in self.running:   # preempted meanwhile
+                continue
+            if len(batch.items) >= self.max_num_seqs or batched + 1 > self.max_num_batched_tokens:
+                break
+            cached = seq.num_cached_tokens
+            preempted_self = False
+            while not mgr.can_cover(seq.id, cached, cached + 1):
+                if self._preempt_one_running(scheduled | {seq.id}):
+                    continue
+                self.running.remove(seq)
+                self.preempt(seq)
+                preempted_self = True
+                break
+            if preempted_self:
+                continue
+            mgr.cover(seq.id, cached, cached + 1)
+            batch.items.append(ScheduledItem(seq, 1, cached, True, True))
+            scheduled.add(seq.id)
+            batched += 1
+
+        # ---- unfinished prompts among the running requests
+        for seq in list(self.running):
+            if not seq.is_partial_prefill or seq.id in scheduled or seq not in self.running:
+                continue
+            if len(batch.items) >= self.max_num_seqs:
+                break
+            remaining = seq.num_tokens - seq.num_cached_tokens
+            if 0 < self.long_prefill_token_threshold < remaining:
+                remaining = self.long_prefill_token_threshold
+            chunk = self._chunked_prefill_size(remaining, self.max_num_batched_tokens - batched, batched)
+            if chunk <= 0:
+                break
+            cached = seq.num_cached_tokens
+            if not mgr.can_cover(seq.id, cached, cached + chunk, seq.num_tokens):
+                # only a window group can be short here; wait for pages rather than evict
+                break
+            mgr.cover(seq.id, cached, cached + chunk, seq.num_tokens)
+            batch.items.append(ScheduledItem(seq, chunk, cached, False, cached + chunk >= seq.num_tokens))
+            scheduled.add(seq.id)
+            batched += chunk
+
+        # ---- new requests, in arrival order
+        now = time.time()
+        while (self.waiting and len(batch.items) < self.max_num_seqs and batched < self.max_num_batched_tokens
+               and self._passed_delay(now)):
+            seq = self.waiting.popleft()
+            if seq.status == SequenceStatus.ABORTED:
+                seq.leave_reason = "aborted"
+                seq.leave_time = time.time()
+                self._rejected.append(seq)
+                continue
+            reason = self._unschedulable_reason(seq)
+            if reason is not None:
+                seq.status = SequenceStatus.FINISHED
+                seq.leave_reason = f"unschedulable: {reason}"
+                seq.leave_time = time.time()
+                self._rejected.append(seq)
+                continue
+            if len(self.running) >= self.max_num_seqs or not mgr.can_open():
+                self.waiting.appendleft(seq)
+                break
+            num_new = seq.num_tokens
+            if self.enable_chunked_prefill and 0 < self.long_prefill_token_threshold < num_new:
+                num_new = self.long_prefill_token_threshold
+            chunk = self._prefill_chunk_for_budget(num_new, self.max_num_batched_tokens - batched, batched)
+            if chunk is None or not mgr.can_cover(seq.id, 0, chunk, seq.num_tokens):
+                self.waiting.appendleft(seq)
+                break
+            self.core.open(seq.id)
+            mgr.cover(seq.id, 0, chunk, seq.num_tokens)
+            seq.status = SequenceStatus.RUNNING
+            seq.num_cached_tokens = 0
+            self.running.append(seq)
+            batch.items.append(ScheduledItem(seq, chunk, 0, False, chunk >= seq.num_tokens))
+            scheduled.add(seq.id)
+            batched += chunk
+
+        if not batch.items:
+            return None
+        if batch.num_prefill:
+            self._last_prompt_time = now
+        return batch
+
+    # ------------------------------------------------------------------ after the step
+
+    def _finish_reason(self, seq: Sequence, token: int) -> str | None:
+        """atom/model_engine/scheduler.py:2296-2329: stop sequences first; only if none matched,
+        eos, then stop token ids, then max_tokens."""
+        for stop_seq in seq.stop_token_sequences:
+            n = len(stop_seq)
+            if n and seq.num_completion_tokens >= 1 and seq.token_ids[-n:] == list(stop_seq):
+                return "stop_sequence"
+        if not seq.ignore_eos and token == self.eos_token_id:
+            return "eos"
+        if not seq.ignore_eos and token in self.stop_token_ids:
+            return f"stop_{token}"
+        if seq.num_completion_tokens >= seq.max_tokens:
+            return "max_tokens"
+        if seq.num_tokens >= self.max_model_len:
+            return "max_model_len"
+        return None
+
+    def postprocess(self, batch: ScheduledBatch, sampled: dict[int, int], step_seconds: float = 0.0) -> list[Sequence]:
+        """``sampled`` maps sequence id -> sampled token for every final item.  Returns the
+        sequences that finished."""
+        finished = []
+        now = time.time()
+        if batch.num_prefill:
+            self._last_prompt_latency = step_seconds
+        for it in batch.items:
+            seq = it.seq
+            seq.num_cached_tokens = it.start + it.num_tokens
+            if not it.is_final:
+                seq.is_partial_prefill = True
+                continue
+            seq.is_partial_prefill = False
+            token = sampled[seq.id]
+            seq.append_token(token)
+            if seq.first_token_time == 0.0:
+                seq.first_token_time = now
+            reason = self._finish_reason(seq, token)
+            if reason is not None:
+                seq.status = SequenceStatus.FINISHED
+                seq.leave_reason = reason
+                seq.leave_time = now
+                self.core.close(seq.id)
+                self.running.remove(seq)
+                finished.append(seq)
+        return finished
