@@ -56,7 +56,7 @@ class LLMEngine:
             from ..config.registry import build_model
             from ..weights.random_init import RandomSource
 
-            source = RandomSource(build_model(cfg.model_config), cfg.seed)
+            source = RandomSource(build_model(cfg.model_config), cfg.seed, device=cfg.device)
         self.model, _ = load_model(cfg.model, dtype=self.dtype, device=cfg.device, model_config=cfg.model_config,
                                    source=source)
         self.core = build_core(

@@ -22,21 +22,17 @@ from ..config.registry import build_model
 from .loader import DictSource, TensorSource, expected_tensors
 
 
-def _generator(seed: int, name: str) -> torch.Generator:
-    g = torch.Generator(device="cpu")
-    g.manual_seed((int(seed) * 1000003 + zlib.crc32(name.encode())) % (2 ** 63))
-    return g
-
-
 def random_tensor(name: str, shape, init: str, seed: int, std: float, norm_std: float,
-                  dtype: torch.dtype) -> torch.Tensor:
-    g = _generator(seed, name)
+                  dtype: torch.dtype, device: str = "cpu") -> torch.Tensor:
+    """Drawn on ``device``; the values depend on (seed, name, device kind) only."""
+    g = torch.Generator(device=device)
+    g.manual_seed((int(seed) * 1000003 + zlib.crc32(name.encode())) % (2 ** 63))
     if init == "zeros":
-        t = torch.zeros(shape)
+        t = torch.zeros(shape, device=device)
     elif init == "one_plus_normal":
-        t = 1.0 + norm_std * torch.randn(shape, generator=g)
+        t = 1.0 + norm_std * torch.randn(shape, generator=g, device=device)
     elif init == "normal":
-        t = std * torch.randn(shape, generator=g)
+        t = torch.randn(shape, generator=g, device=device, dtype=torch.float32 if device == "cpu" else dtype) * std
     else:
         raise ValueError(f"unknown init {init!r}")
     return t.to(dtype)
@@ -46,9 +42,10 @@ class RandomSource(TensorSource):
     """Draws each tensor when it is asked for (nothing is held: an 8B model streams through)."""
 
     def __init__(self, model, seed: int, std: float = 0.02, norm_std: float = 0.1,
-                 dtype: torch.dtype = torch.bfloat16):
+                 dtype: torch.dtype = torch.bfloat16, device: str = "cpu"):
         self.expected = expected_tensors(model)
         self.seed, self.std, self.norm_std, self._dtype = seed, std, norm_std, dtype
+        self.device = device
         self.where = f"<random weights, seed {seed}>"
 
     def names(self):
@@ -63,7 +60,7 @@ class RandomSource(TensorSource):
     def get(self, name):
         shape, spec = self.expected[name]
         init = "normal" if spec.init == "normal" else spec.init
-        return random_tensor(name, shape, init, self.seed, self.std, self.norm_std, self._dtype)
+        return random_tensor(name, shape, init, self.seed, self.std, self.norm_std, self._dtype, self.device)
 
 
 def random_state_dict(config: ModelConfig, seed: int, std: float = 0.02, norm_std: float = 0.1,
