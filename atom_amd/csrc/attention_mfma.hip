@@ -1,0 +1,362 @@
+// Paged attention on the matrix cores (bfloat16 in, float32 accumulate), gfx950.
+//
+// One wave is one work item; it owns up to 16 * RT query rows and walks its keys 16 at a
+// time.  Both products are formed transposed so that a lane always holds values of ONE
+// query row (row = lane % 16):
+//
+//     S^T[key][row] = K[key][:] . Q[row][:]        A = K rows (from the key pages),  B = Q
+//     O^T[d][row]   = V^T[d][key] . P[row][key]    A = V^T rows (value pages are stored
+//                                                  transposed, keys contiguous),     B = P
+//
+// The first product leaves lane (row, g = lane / 16) with the scores of keys 4g..4g+3 of
+// the block, which is exactly the B operand of the second, so probabilities never move
+// between lanes, and the running maximum, sum and rescale factor of a row are per-lane
+// scalars (the maximum needs two cross-lane exchanges over g).  Softmax is float32, in
+// the exp2 domain.
+//
+// Two modes:
+//   decode   a request's single new token: rows are the query heads that share a KV head;
+//            the visible keys are split over `parts` waves whose partial results (running
+//            maximum, sum, unnormalised output) a second kernel merges.
+//   prefill  a tile of consecutive query tokens of one head; causal by absolute position
+//            (a portion of a prompt sees the cached keys before it), optional window.
+//
+// Pages: keys [num_pages, Hkv, page_size, D]; values [num_pages, Hkv, D, page_size];
+// page_size a multiple of 4.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+
+struct AttnParams {
+  const bf16_t* q;        // [tokens, Hq, D]
+  const bf16_t* k_cache;
+  const bf16_t* v_cache;
+  bf16_t* out;            // [tokens, Hq, D]
+  const int* cu_q;        // [num_seqs + 1]
+  const int* ctx_lens;    // [num_seqs]
+  const int* block_tables;  // [num_seqs, max_blocks]
+  const int* tiles;       // prefill: [num_tiles, 2] = (request, first row of the tile within its tokens)
+  float* ws_o;            // decode: [seqs, Hq, parts, D]
+  float* ws_ml;           // decode: [seqs, Hq, parts, 2]
+  int max_blocks, hq, hkv, page_size, window, seq_offset, parts;
+  float scale_log2;       // softmax scale * log2(e)
+};
+
+__device__ __forceinline__ s16x4 as_s16x4(bf16x4 v) { return __builtin_bit_cast(s16x4, v); }
+
+template <int D, int RT, bool DECODE>
+__global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
+  constexpr bool KX32 = (D % 32 == 0);
+  constexpr int KCH = KX32 ? D / 32 : D / 16;  // K/Q register chunks
+  constexpr int DT = D / 16;                   // output tiles along d
+  const int lane = threadIdx.x;
+  const int r16 = lane & 15;
+  const int g = lane >> 4;
+  const int group = p.hq / p.hkv;
+
+  int seq, kvh, head0, nrows, tok0, pos0, part = 0;
+  int ctx;
+  if (DECODE) {
+    seq = blockIdx.z + p.seq_offset;
+    kvh = blockIdx.y;
+    part = blockIdx.x;
+    ctx = p.ctx_lens[seq];
+    head0 = kvh * group;
+    nrows = group;            // rows are heads head0 .. head0 + group - 1 of one token
+    tok0 = p.cu_q[seq];
+    pos0 = ctx - 1;
+  } else {
+    const int tile = blockIdx.x;
+    seq = p.tiles[2 * tile];
+    const int row_start = p.tiles[2 * tile + 1];
+    head0 = blockIdx.y;
+    kvh = head0 / group;
+    ctx = p.ctx_lens[seq];
+    const int q_begin = p.cu_q[seq];
+    const int q_len = p.cu_q[seq + 1] - q_begin;
+    nrows = min(16 * RT, q_len - row_start);
+    tok0 = q_begin + row_start;
+    pos0 = ctx - q_len + row_start;   // absolute position of the tile's first row
+  }
+  const int* table = p.block_tables + (size_t)seq * p.max_blocks;
+  const int ps = p.page_size;
+
+  // ---- key range of this work item
+  int kb, ke;
+  if (DECODE) {
+    int vis = 0;
+    if (p.window > 0 && ctx - p.window > 0) vis = (ctx - p.window) & ~15;
+    const int len = ctx - vis;
+    int chunk = (len + p.parts - 1) / p.parts;
+    chunk = (chunk + 15) & ~15;
+    kb = vis + part * chunk;
+    ke = min(ctx, kb + chunk);
+  } else {
+    kb = 0;
+    if (p.window > 0 && pos0 - p.window + 1 > 0) kb = (pos0 - p.window + 1) & ~15;
+    ke = pos0 + nrows;   // one past the last row's own position
+  }
+
+  // ---- per-lane row data
+  int row_pos[RT];
+  bool row_ok[RT];
+  bf16x8 q32[RT][KX32 ? KCH : 1];
+  s16x4 q16[RT][KX32 ? 1 : KCH];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = rt * 16 + r16;
+    row_ok[rt] = row < nrows;
+    const bf16_t* qr;
+    if (DECODE) {
+      row_pos[rt] = pos0;
+      qr = p.q + ((size_t)tok0 * p.hq + head0 + row) * D;
+    } else {
+      row_pos[rt] = pos0 + row;
+      qr = p.q + ((size_t)(tok0 + row) * p.hq + head0) * D;
+    }
+    if (KX32) {
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) {
+        bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (row_ok[rt]) v = *reinterpret_cast<const bf16x8*>(qr + 32 * j + 8 * g);
+        q32[rt][j] = v;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) {
+        s16x4 v = {0, 0, 0, 0};
+        if (row_ok[rt]) v = *reinterpret_cast<const s16x4*>(qr + 16 * j + 4 * g);
+        q16[rt][j] = v;
+      }
+    }
+  }
+
+  f32x4 acc[RT][DT];
+  float run_max[RT], run_sum[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    run_max[rt] = -INFINITY;
+    run_sum[rt] = 0.f;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) acc[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int k0 = kb; k0 < ke; k0 += 16) {
+    // ---- K block: this lane's key row is k0 + r16 (clamped into the context for addressing)
+    const int krow = min(k0 + r16, ke - 1);
+    const int kpage = table[krow / ps];
+    const bf16_t* kptr = p.k_cache + (((size_t)kpage * p.hkv + kvh) * ps + (krow % ps)) * D;
+    // ---- V block: this lane's keys are k0 + 4g .. + 3, of output rows d = 16 t + r16
+    const int vkey = min(k0 + 4 * g, ((ke - 1) & ~3));
+    const int vpage = table[vkey / ps];
+    const bf16_t* vptr = p.v_cache + (((size_t)vpage * p.hkv + kvh) * D + r16) * (size_t)ps + (vkey % ps);
+
+    f32x4 s[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) s[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (KX32) {
+      bf16x8 kreg[KX32 ? KCH : 1];
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) kreg[j] = *reinterpret_cast<const bf16x8*>(kptr + 32 * j + 8 * g);
+#pragma unroll
+      for (int j = 0; j < KCH; ++j)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          s[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[j], q32[rt][j], s[rt], 0, 0, 0);
+    } else {
+      s16x4 kreg[KX32 ? 1 : KCH];
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) kreg[j] = *reinterpret_cast<const s16x4*>(kptr + 16 * j + 4 * g);
+#pragma unroll
+      for (int j = 0; j < KCH; ++j)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          s[rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[j], q16[rt][j], s[rt], 0, 0, 0);
+    }
+    s16x4 vreg[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) vreg[t] = *reinterpret_cast<const s16x4*>(vptr + (size_t)(16 * t) * ps);
+
+    // ---- softmax update per row tile; lane holds keys k0 + 4g + i of row r16
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float sc[4];
+      float mx = -INFINITY;
+      const int hi = min(row_pos[rt], ke - 1);                        // last visible key
+      const int lo = p.window > 0 ? row_pos[rt] - p.window + 1 : 0;   // first visible key
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = k0 + 4 * g + i;
+        const bool vis = key <= hi && key >= lo && key >= kb;
+        sc[i] = vis ? s[rt][i] * p.scale_log2 : -INFINITY;
+        mx = fmaxf(mx, sc[i]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float new_max = fmaxf(run_max[rt], mx);
+      const float base = new_max == -INFINITY ? 0.f : new_max;
+      const float alpha = exp2f(run_max[rt] - base);   // 0 while nothing was seen yet
+      float psum = 0.f;
+      bf16x4 pb;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = exp2f(sc[i] - base);
+        psum += pv;
+        pb[i] = static_cast<bf16_t>(pv);
+      }
+      run_sum[rt] = run_sum[rt] * alpha + psum;
+      run_max[rt] = new_max;
+      const s16x4 pbits = as_s16x4(pb);
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        f32x4 a = acc[rt][t];
+        a[0] *= alpha; a[1] *= alpha; a[2] *= alpha; a[3] *= alpha;
+        acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg[t], pbits, a, 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- write: lane holds O[row r16][d = 16 t + 4 g + i]
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    float total = run_sum[rt];
+    total += __shfl_xor(total, 16, kWave);
+    total += __shfl_xor(total, 32, kWave);
+    if (!row_ok[rt]) continue;
+    const int row = rt * 16 + r16;
+    if (DECODE && p.parts > 1) {
+      const size_t slot = ((size_t)(blockIdx.z * p.hq + head0 + row)) * p.parts + part;
+      float* wo = p.ws_o + slot * D;
+#pragma unroll
+      for (int t = 0; t < DT; ++t) *reinterpret_cast<f32x4*>(wo + 16 * t + 4 * g) = acc[rt][t];
+      if (g == 0) {
+        p.ws_ml[slot * 2] = run_max[rt];
+        p.ws_ml[slot * 2 + 1] = total;
+      }
+    } else {
+      bf16_t* dst = DECODE ? p.out + ((size_t)tok0 * p.hq + head0 + row) * D
+                           : p.out + ((size_t)(tok0 + row) * p.hq + head0) * D;
+      const float inv = total > 0.f ? 1.f / total : 0.f;
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        bf16x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = static_cast<bf16_t>(acc[rt][t][i] * inv);
+        *reinterpret_cast<bf16x4*>(dst + 16 * t + 4 * g) = o;
+      }
+    }
+  }
+}
+
+// Merges the partial results of a decode row: one block per (request, head), one thread per d.
+__global__ void attention_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+                                       bf16_t* __restrict__ out, const int* __restrict__ cu_q, int seq_offset,
+                                       int hq, int d, int parts) {
+  const int seq = blockIdx.y;
+  const int head = blockIdx.x;
+  const size_t base = ((size_t)seq * hq + head) * parts;
+  float top = -INFINITY;
+  for (int k = 0; k < parts; ++k) top = fmaxf(top, ws_ml[(base + k) * 2]);
+  const int tok = cu_q[seq + seq_offset];
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float num = 0.f, den = 0.f;
+    for (int k = 0; k < parts; ++k) {
+      const float m = ws_ml[(base + k) * 2];
+      if (m == -INFINITY) continue;
+      const float w = exp2f(m - top);
+      num += w * ws_o[(base + k) * d + i];
+      den += w * ws_ml[(base + k) * 2 + 1];
+    }
+    out[((size_t)tok * hq + head) * d + i] = static_cast<bf16_t>(den > 0.f ? num / den : 0.f);
+  }
+}
+
+template <int D>
+static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
+  const int group = p.hq / p.hkv;
+  dim3 grid(p.parts, p.hkv, seqs), block(kWave);
+  if (group <= 16) hipLaunchKernelGGL((attention_mfma_kernel<D, 1, true>), grid, block, 0, stream, p);
+  else if (group <= 32) hipLaunchKernelGGL((attention_mfma_kernel<D, 2, true>), grid, block, 0, stream, p);
+  else return ATOM_UNSUPPORTED;
+  if (p.parts > 1)
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(p.hq, seqs), dim3(D >= 128 ? 128 : 64), 0, stream, p.ws_o,
+                       p.ws_ml, p.out, p.cu_q, p.seq_offset, p.hq, D, p.parts);
+  return launch_status();
+}
+
+template <int D>
+static int launch_prefill(const AttnParams& p, int num_tiles, int rows_per_tile, hipStream_t stream) {
+  dim3 grid(num_tiles, p.hq), block(kWave);
+  if (rows_per_tile == 16) hipLaunchKernelGGL((attention_mfma_kernel<D, 1, false>), grid, block, 0, stream, p);
+  else if (rows_per_tile == 32) hipLaunchKernelGGL((attention_mfma_kernel<D, 2, false>), grid, block, 0, stream, p);
+  else return ATOM_BAD_SHAPE;
+  return launch_status();
+}
+
+#define ATOM_FOR_HEAD_DIM(d, CALL)        \
+  switch (d) {                            \
+    case 16: CALL(16); break;             \
+    case 32: CALL(32); break;             \
+    case 64: CALL(64); break;             \
+    case 96: CALL(96); break;             \
+    case 128: CALL(128); break;           \
+    case 256: CALL(256); break;           \
+    default: return ATOM_UNSUPPORTED;     \
+  }
+
+// 1 if this head size has a matrix-core kernel.
+ATOM_EXPORT int atom_attention_mfma_supports(int d, int page_size, int group) {
+  if (page_size % 4 || group > 32) return 0;
+  return d == 16 || d == 32 || d == 64 || d == 96 || d == 128 || d == 256;
+}
+
+static int check_common(int hq, int hkv, int d, int page_size, int max_blocks) {
+  if (hq <= 0 || hkv <= 0 || hq % hkv || d <= 0 || page_size <= 0 || page_size % 4 || max_blocks <= 0)
+    return ATOM_BAD_SHAPE;
+  if (hq > 65535) return ATOM_TOO_LARGE;
+  return ATOM_OK;
+}
+
+// Decode: requests seq_offset .. seq_offset + seqs - 1 each bring one new token (row cu_q[seq]).
+// ws_o needs seqs * hq * parts * d floats, ws_ml seqs * hq * parts * 2 (unused when parts == 1).
+ATOM_EXPORT int atom_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                      const int* cu_q, const int* ctx_lens, const int* block_tables, int max_blocks,
+                                      int seq_offset, int seqs, int hq, int hkv, int d, int page_size, float scale,
+                                      int window, int parts, float* ws_o, float* ws_ml, hipStream_t stream) {
+  if (int st = check_common(hq, hkv, d, page_size, max_blocks)) return st;
+  if (seqs < 0 || parts < 1 || seq_offset < 0) return ATOM_BAD_SHAPE;
+  if (parts > 1 && (!ws_o || !ws_ml)) return ATOM_BAD_SHAPE;
+  if (seqs > 65535 || hkv > 65535) return ATOM_TOO_LARGE;
+  if (seqs == 0) return ATOM_OK;
+  AttnParams p{};
+  p.q = (const bf16_t*)q; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache;
+  p.out = (bf16_t*)out; p.cu_q = cu_q; p.ctx_lens = ctx_lens; p.block_tables = block_tables; p.tiles = nullptr;
+  p.ws_o = ws_o; p.ws_ml = ws_ml; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
+  p.window = window; p.seq_offset = seq_offset; p.parts = parts; p.scale_log2 = scale * 1.4426950408889634f;
+#define CALL(DD) return launch_decode<DD>(p, seqs, stream)
+  ATOM_FOR_HEAD_DIM(d, CALL)
+#undef CALL
+  return ATOM_OK;
+}
+
+// Prefill: `tiles` lists (request, first row) for every tile of `rows_per_tile` (16 or 32) query tokens.
+ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                       const int* cu_q, const int* ctx_lens, const int* block_tables, int max_blocks,
+                                       const int* tiles, int num_tiles, int rows_per_tile, int hq, int hkv, int d,
+                                       int page_size, float scale, int window, hipStream_t stream) {
+  if (int st = check_common(hq, hkv, d, page_size, max_blocks)) return st;
+  if (num_tiles < 0 || !tiles) return ATOM_BAD_SHAPE;
+  if (num_tiles == 0) return ATOM_OK;
+  AttnParams p{};
+  p.q = (const bf16_t*)q; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache;
+  p.out = (bf16_t*)out; p.cu_q = cu_q; p.ctx_lens = ctx_lens; p.block_tables = block_tables; p.tiles = tiles;
+  p.ws_o = nullptr; p.ws_ml = nullptr; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
+  p.window = window; p.seq_offset = 0; p.parts = 1; p.scale_log2 = scale * 1.4426950408889634f;
+#define CALL(DD) return launch_prefill<DD>(p, num_tiles, rows_per_tile, stream)
+  ATOM_FOR_HEAD_DIM(d, CALL)
+#undef CALL
+  return ATOM_OK;
+}

@@ -152,7 +152,15 @@ class EngineCore:
         want = [row_of_entry[i] + w for i, e in enumerate(entries) for w in e.want]
         want_rows = np.asarray(want, dtype=np.int32)
 
-        pieces = [tokens, positions, token_seq, starts, context_lens, want_rows]
+        # tiles of query rows for the prompt portions (requests with more than one token come
+        # first); the tiles with the most keys are listed first
+        num_prefill = sum(1 for n in q_lens if n > 1)
+        rows_per_tile = 32 if max(q_lens) > 16 else 16
+        tile_list = [(b, r0) for b in range(num_prefill) for r0 in range(0, q_lens[b], rows_per_tile)]
+        tile_list.sort(key=lambda t: -(cached[t[0]] + t[1]))
+        tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1)
+
+        pieces = [tokens, positions, token_seq, starts, context_lens, want_rows, tiles]
         group_shapes = []
         for gi, g in enumerate(mgr.groups):
             tables = [mgr.block_table(entries[i].req_id, gi) for i in order]
@@ -179,18 +187,20 @@ class EngineCore:
         def view(k):
             return dev[offsets[k]:offsets[k] + pieces[k].size]
 
-        d_tokens, d_positions, d_token_seq, d_starts, d_ctx, d_want = (view(k) for k in range(6))
+        d_tokens, d_positions, d_token_seq, d_starts, d_ctx, d_want, d_tiles = (view(k) for k in range(7))
+        first_group = 7
         ctx = StepContext(ops=self.ops, dtype=self.dtype, device=self.device, num_tokens=total, num_seqs=num_seqs,
                           positions=d_positions, seq_starts=[int(s) for s in starts[:-1]], seq_lens=q_lens,
                           seq_cached=cached,
                           state_slots=[mgr.state_slot(entries[i].req_id) for i in order])
         for gi, g in enumerate(mgr.groups):
-            bt = view(6 + 2 * gi).view(num_seqs, group_shapes[gi])
+            bt = view(first_group + 2 * gi).view(num_seqs, group_shapes[gi])
             ctx.attention[gi] = AttentionMeta(
                 token_seq=d_token_seq, positions=d_positions, block_tables=bt, cu_seqlens_q=d_starts,
                 context_lens=d_ctx, num_seqs=num_seqs, num_tokens=total, max_q_len=max(q_lens),
-                max_context_len=int(context_lens.max()), page_size=g.page_size)
-            ctx.slot_mappings[gi] = view(7 + 2 * gi)
+                max_context_len=int(context_lens.max()), page_size=g.page_size, num_prefill=num_prefill,
+                prefill_tiles=d_tiles.view(-1, 2) if num_prefill else None, rows_per_tile=rows_per_tile)
+            ctx.slot_mappings[gi] = view(first_group + 1 + 2 * gi)
         return ctx, d_tokens, (d_want if want_rows.size else None)
 
 

@@ -53,6 +53,11 @@ class AttentionMeta:
     max_q_len: int
     max_context_len: int
     page_size: int
+    # requests 0 .. num_prefill-1 bring more than one token (prompt portions), the rest one each;
+    # prefill_tiles [num_tiles, 2] lists (request, first row) of every tile of rows_per_tile rows
+    num_prefill: int = 0
+    prefill_tiles: torch.Tensor | None = None
+    rows_per_tile: int = 16
 
 
 def _ptr(t: torch.Tensor | None):
@@ -76,9 +81,27 @@ class HipKernels:
             raise KernelError(f"could not load the kernel library {path}: {e}") from e
         self.path = path
         for fn in ("atom_embedding", "atom_rmsnorm", "atom_silu_mul", "atom_qk_norm_rope_kv_write",
-                   "atom_paged_attention_generic", "atom_gemm_f32", "atom_sample", "atom_exponential_noise"):
+                   "atom_paged_attention_generic", "atom_gemm_f32", "atom_sample", "atom_exponential_noise",
+                   "atom_attention_mfma_supports", "atom_attention_decode", "atom_attention_prefill"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
+        self.use_mfma_attention = True
+        self._ws: dict[str, torch.Tensor] = {}
+        self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
+
+    def workspace(self, name: str, numel: int, dtype=torch.float32) -> torch.Tensor:
+        """A scratch tensor that only grows; one per name."""
+        t = self._ws.get(name)
+        if t is None or t.numel() < numel or t.dtype != dtype:
+            t = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
+            self._ws[name] = t
+        return t
+
+    def decode_parts(self, seqs: int, hkv: int, max_context: int) -> int:
+        """Over how many waves a decode row's keys are split: enough waves to fill the chip,
+        at least 64 keys each."""
+        want = -(-8 * self.num_cus // max(1, seqs * hkv))
+        return max(1, min(want, 64, -(-max_context // 64)))
 
     # ------------------------------------------------------------------ helpers
 
@@ -182,8 +205,40 @@ class HipKernels:
             self._stream()))
         return q_out
 
+    def _attention_mfma(self, q, k_cache, v_cache, out, meta, scale, window, parts=None):
+        tokens, hq, d = q.shape
+        _, hkv, page_size, _ = k_cache.shape
+        self._check("cu_seqlens_q", meta.cu_seqlens_q, torch.int32, (meta.num_seqs + 1,))
+        self._check("context_lens", meta.context_lens, torch.int32, (meta.num_seqs,))
+        bt = meta.block_tables
+        if bt.shape[0] != meta.num_seqs:
+            raise KernelError("attention: one block table row per request is needed")
+        if meta.num_prefill:
+            tiles = meta.prefill_tiles
+            self._check("prefill tiles", tiles, torch.int32, (None, 2))
+            if meta.rows_per_tile not in (16, 32):
+                raise KernelError("attention: tiles hold 16 or 32 rows")
+            self._done("attention_prefill", self.lib.atom_attention_prefill(
+                _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.cu_seqlens_q), _ptr(meta.context_lens),
+                _ptr(bt), bt.shape[1], _ptr(tiles), tiles.shape[0], meta.rows_per_tile, hq, hkv, d, page_size,
+                ctypes.c_float(scale), int(window or 0), self._stream()))
+        seqs = meta.num_seqs - meta.num_prefill
+        if seqs:
+            if parts is None:
+                visible = min(meta.max_context_len, window) if window else meta.max_context_len
+                parts = self.decode_parts(seqs, hkv, visible)
+            ws_o = ws_ml = None
+            if parts > 1:
+                ws_o = self.workspace("attn_o", seqs * hq * parts * d)
+                ws_ml = self.workspace("attn_ml", seqs * hq * parts * 2)
+            self._done("attention_decode", self.lib.atom_attention_decode(
+                _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.cu_seqlens_q), _ptr(meta.context_lens),
+                _ptr(bt), bt.shape[1], meta.num_prefill, seqs, hq, hkv, d, page_size, ctypes.c_float(scale),
+                int(window or 0), parts, _ptr(ws_o), _ptr(ws_ml), self._stream()))
+        return out
+
     def paged_attention(self, q, k_cache, v_cache, out, meta: AttentionMeta, scale: float,
-                        window: int | None = None):
+                        window: int | None = None, parts: int | None = None):
         tokens, hq, d = q.shape
         _, hkv, page_size, _ = k_cache.shape
         dt = q.dtype
@@ -200,6 +255,10 @@ class HipKernels:
             raise KernelError("attention: the batch's page size differs from the cache's")
         if meta.max_context_len > meta.block_tables.shape[1] * page_size:
             raise KernelError("attention: a context is longer than its block table can name")
+        group = hq // hkv
+        if (dt == torch.bfloat16 and self.use_mfma_attention
+                and self.lib.atom_attention_mfma_supports(d, page_size, group)):
+            return self._attention_mfma(q, k_cache, v_cache, out, meta, scale, window, parts)
         self._done("paged_attention", self.lib.atom_paged_attention_generic(
             _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.token_seq), _ptr(meta.positions),
             _ptr(meta.block_tables), meta.block_tables.shape[1], self._code(q), tokens, hq, hkv, d, page_size,

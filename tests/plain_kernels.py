@@ -69,7 +69,7 @@ class PlainKernels:
                 v_cache[page, :, :, off] = v[i].to(v_cache.dtype)
         return q_out
 
-    def paged_attention(self, q, k_cache, v_cache, out, meta, scale, window=None):
+    def paged_attention(self, q, k_cache, v_cache, out, meta, scale, window=None, parts=None):
         tokens, hq, d = q.shape
         page_size = k_cache.shape[2]
         for t in range(tokens):

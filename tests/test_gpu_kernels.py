@@ -1,0 +1,359 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the engine's:
+widths and vocabularies that are no power of two, head sizes in steps of 16, odd numbers
+of heads and groups, several page sizes."""
+
+import math
+
+import pytest
+import torch
+
+from helpers import gpu_ops
+from plain_kernels import PlainKernels, exponential_noise_row
+from atom_amd.kernels.hip import AttentionMeta, KernelError
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+PLAIN = PlainKernels()
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def close(got, want, dtype, scale=None):
+    got, want = got.detach().cpu().double(), want.detach().cpu().double()
+    scale = scale or max(1e-6, float(want.abs().max()))
+    tol = 2e-6 if dtype == torch.float32 else 1.2e-2   # a few ulp of the output's type
+    worst = float((got - want).abs().max())
+    assert worst <= tol * scale, f"max diff {worst:.3e} > {tol * scale:.3e}"
+
+
+@pytest.mark.parametrize("tdtype", DTYPES)
+@pytest.mark.parametrize("odtype", DTYPES)
+def test_embedding(tdtype, odtype):
+    table = rnd((311, 136), tdtype, 0)
+    ids = torch.tensor([0, 310, 5, 5, 17, 200], dtype=torch.int32)
+    out = torch.empty((6, 136), dtype=odtype, device=DEV)
+    gpu_ops().embedding(table.to(DEV), ids.to(DEV), out)
+    want = torch.empty((6, 136), dtype=odtype)
+    PLAIN.embedding(table, ids, want)
+    assert torch.equal(out.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [16, 136, 4096, 5000])
+@pytest.mark.parametrize("mode", ["plain", "init", "add"])
+def test_rmsnorm(dtype, width, mode):
+    rows = 7
+    x = rnd((rows, width), dtype, 1, 3.0)
+    w = 1 + rnd((width,), torch.float32, 2, 0.2)
+    res = rnd((rows, width), torch.float32, 3, 2.0)
+    out = torch.empty_like(x, device=DEV)
+    res_gpu = res.to(DEV)
+    gpu_ops().rmsnorm(x.to(DEV), w.to(DEV), 1e-5, out, residual=res_gpu if mode != "plain" else None, mode=mode)
+    want = torch.empty_like(x)
+    res_want = res.clone()
+    PLAIN.rmsnorm(x, w, 1e-5, want, residual=res_want if mode != "plain" else None, mode=mode)
+    close(out, want, dtype)
+    if mode != "plain":
+        close(res_gpu, res_want, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_rows(dtype):
+    x = rnd((9, 200), dtype, 4)
+    res = rnd((9, 200), torch.float32, 5)
+    w = 1 + rnd((200,), torch.float32, 6, 0.3)
+    rows = torch.tensor([8, 0, 3], dtype=torch.int32)
+    out = torch.empty((3, 200), dtype=dtype, device=DEV)
+    res_gpu = res.to(DEV)
+    gpu_ops().rmsnorm(x.to(DEV), w.to(DEV), 1e-6, out, residual=res_gpu, mode="add", rows=rows.to(DEV))
+    want = torch.empty((3, 200), dtype=dtype)
+    PLAIN.rmsnorm(x, w, 1e-6, want, residual=res.clone(), mode="add", rows=rows)
+    close(out, want, dtype)
+    assert torch.equal(res_gpu.cpu(), res), "the residual stream must stay as it was"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(dtype):
+    x = rnd((5, 2 * 333), dtype, 7, 2.0)
+    out = torch.empty((5, 333), dtype=dtype, device=DEV)
+    gpu_ops().silu_mul(x.to(DEV), out)
+    want = torch.empty((5, 333), dtype=dtype)
+    PLAIN.silu_mul(x, want)
+    close(out, want, dtype)
+    swapped = torch.cat((x[:, 333:], x[:, :333]), dim=1)
+    other = torch.empty((5, 333), dtype=dtype)
+    PLAIN.silu_mul(swapped, other)
+    assert (other.float() - want.float()).abs().max() > 0.1, "gate and up must not be interchangeable"
+
+
+@pytest.mark.parametrize("xd,wd", [(torch.float32, torch.float32), (torch.bfloat16, torch.float32),
+                                   (torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("m,n,k", [(1, 311, 96), (7, 64, 130), (70, 200, 65), (3, 1, 17)])
+def test_gemm_f32_kernel(xd, wd, m, n, k):
+    ops = gpu_ops()
+    x, w, b = rnd((m, k), xd, 8), rnd((n, k), wd, 9), rnd((n,), torch.float32, 10)
+    ops.allow_library_gemm = False
+    try:
+        y = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), out_dtype=torch.float32)
+    finally:
+        ops.allow_library_gemm = True
+    want = PLAIN.linear(x, w, b, out_dtype=torch.float32)
+    close(y, want, torch.float32, scale=float(want.abs().max()) * 2)
+
+
+def test_gemm_f32_rows_do_not_depend_on_batch():
+    ops = gpu_ops()
+    x, w = rnd((70, 300), torch.float32, 11).to(DEV), rnd((129, 300), torch.float32, 12).to(DEV)
+    whole = ops.linear(x, w)
+    for lo, hi in ((0, 1), (5, 6), (63, 70), (10, 40)):
+        assert torch.equal(ops.linear(x[lo:hi].contiguous(), w), whole[lo:hi])
+
+
+def test_linear_bf16_library_path():
+    ops = gpu_ops()
+    x, w, b = rnd((33, 136), torch.bfloat16, 13), rnd((517, 136), torch.bfloat16, 14), rnd((517,), torch.float32, 15)
+    y = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV))
+    close(y, PLAIN.linear(x, w, b), torch.bfloat16)
+    y32 = ops.linear(x.to(DEV), w.to(DEV), None, out_dtype=torch.float32)
+    assert y32.dtype == torch.float32
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,d,rot,page", [(4, 2, 16, 16, 16), (6, 3, 32, 32, 8), (5, 5, 48, 24, 4),
+                                              (8, 1, 128, 128, 32), (3, 1, 80, 0, 16)])
+@pytest.mark.parametrize("norm", [True, False])
+def test_qk_norm_rope_kv_write(dtype, hq, hkv, d, rot, page, norm):
+    tokens, pages, max_pos = 11, 6, 50
+    qkv = rnd((tokens, (hq + 2 * hkv) * d), dtype, 16, 2.0)
+    qw = 1 + rnd((d,), torch.float32, 17, 0.2) if norm else None
+    kw = 1 + rnd((d,), torch.float32, 18, 0.2) if norm else None
+    ang = torch.outer(torch.arange(max_pos, dtype=torch.float32), 1.0 / (1e4 ** (torch.arange(0, max(rot, 2), 2) / max(rot, 2))))
+    cos, sin = ang.cos().contiguous(), ang.sin().contiguous()
+    positions = torch.tensor([3, 4, 5, 0, 1, 49, 20, 21, 22, 23, 7], dtype=torch.int32)
+    perm = torch.randperm(pages * page, generator=torch.Generator().manual_seed(19))[:tokens].to(torch.int32)
+    slots = perm.clone()
+    slots[4] = -1   # a padding row writes nothing
+    kc = rnd((pages, hkv, page, d), dtype, 20)
+    vc = rnd((pages, hkv, d, page), dtype, 21)
+    kc_gpu, vc_gpu = kc.to(DEV), vc.to(DEV)
+    q_gpu = torch.empty((tokens, hq, d), dtype=dtype, device=DEV)
+    dev = lambda t: t.to(DEV) if t is not None else None   # noqa: E731
+    gpu_ops().qk_norm_rope_kv_write(qkv.to(DEV), q_gpu, kc_gpu, vc_gpu, dev(qw), dev(kw), cos.to(DEV), sin.to(DEV),
+                                    positions.to(DEV), slots.to(DEV), hq, hkv, d, rot, page, 1e-5)
+    q_want = torch.empty((tokens, hq, d), dtype=dtype)
+    PLAIN.qk_norm_rope_kv_write(qkv, q_want, kc, vc, qw, kw, cos, sin, positions, slots, hq, hkv, d, rot, page, 1e-5)
+    close(q_gpu, q_want, dtype)
+    close(kc_gpu, kc, dtype)
+    close(vc_gpu, vc, dtype)
+    # reading another run's cache: nothing is written
+    before_k, before_v = kc_gpu.clone(), vc_gpu.clone()
+    gpu_ops().qk_norm_rope_kv_write(qkv.to(DEV), q_gpu, kc_gpu, vc_gpu, dev(qw), dev(kw), cos.to(DEV), sin.to(DEV),
+                                    positions.to(DEV), slots.to(DEV), hq, hkv, d, rot, page, 1e-5, write_kv=False)
+    assert torch.equal(before_k, kc_gpu) and torch.equal(before_v, vc_gpu)
+
+
+def _attention_case(dtype, hq, hkv, d, page, window, q_lens, ctx_lens, seed, scale_one=None):
+    """A batch with its cache filled at random pages; returns what both implementations need."""
+    g = torch.Generator().manual_seed(seed)
+    num_seqs = len(q_lens)
+    order = sorted(range(num_seqs), key=lambda i: q_lens[i] == 1)
+    q_lens = [q_lens[i] for i in order]
+    ctx_lens = [ctx_lens[i] for i in order]
+    pages_per = [-(-c // page) for c in ctx_lens]
+    total_pages = sum(pages_per) + 3
+    perm = torch.randperm(total_pages, generator=g).tolist()
+    width = max(pages_per)
+    tables = torch.zeros((num_seqs, width), dtype=torch.int32)
+    at = 0
+    for b, n in enumerate(pages_per):
+        tables[b, :n] = torch.tensor(perm[at:at + n], dtype=torch.int32)
+        at += n
+    kc = (torch.randn((total_pages, hkv, page, d), generator=g)).to(dtype)
+    vc = (torch.randn((total_pages, hkv, d, page), generator=g)).to(dtype)
+    tokens = sum(q_lens)
+    q = (torch.randn((tokens, hq, d), generator=g)).to(dtype)
+    if scale_one is not None:   # make one far key stand out for one query
+        b, key, boost = scale_one
+        pg, off = int(tables[b, key // page]), key % page
+        start = sum(q_lens[:b])
+        for h in range(hq):
+            kc[pg, h // (hq // hkv), off] = (q[start + q_lens[b] - 1, h].float() * boost).to(dtype)
+    cu = [0]
+    for n in q_lens:
+        cu.append(cu[-1] + n)
+    token_seq = torch.tensor([b for b, n in enumerate(q_lens) for _ in range(n)], dtype=torch.int32)
+    positions = torch.tensor([ctx_lens[b] - q_lens[b] + i for b in range(num_seqs) for i in range(q_lens[b])],
+                             dtype=torch.int32)
+    num_prefill = sum(1 for n in q_lens if n > 1)
+    rpt = 32 if max(q_lens) > 16 else 16
+    tiles = torch.tensor([(b, r) for b in range(num_prefill) for r in range(0, q_lens[b], rpt)] or [(0, 0)],
+                         dtype=torch.int32)
+
+    def meta(dev):
+        return AttentionMeta(token_seq=token_seq.to(dev), positions=positions.to(dev), block_tables=tables.to(dev),
+                             cu_seqlens_q=torch.tensor(cu, dtype=torch.int32).to(dev),
+                             context_lens=torch.tensor(ctx_lens, dtype=torch.int32).to(dev), num_seqs=num_seqs,
+                             num_tokens=tokens, max_q_len=max(q_lens), max_context_len=max(ctx_lens), page_size=page,
+                             num_prefill=num_prefill, prefill_tiles=tiles.to(dev) if num_prefill else None,
+                             rows_per_tile=rpt)
+
+    return q, kc, vc, meta
+
+
+ATTN_SHAPES = [  # hq, hkv, d, page
+    (4, 2, 16, 16), (6, 3, 32, 8), (8, 2, 64, 16), (5, 5, 96, 4), (32, 8, 128, 16), (3, 1, 256, 32), (40, 2, 64, 16),
+    (2, 1, 48, 16), (7, 7, 80, 8),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,d,page", ATTN_SHAPES)
+@pytest.mark.parametrize("window", [None, 37])
+def test_paged_attention_mixed_batch(dtype, hq, hkv, d, page, window):
+    q_lens = [33, 2, 1, 1, 70, 1, 16]
+    ctx_lens = [33, 150, 1, 97, 200, 310, 16]
+    q, kc, vc, meta = _attention_case(dtype, hq, hkv, d, page, window, q_lens, ctx_lens, seed=hq * 100 + d)
+    out = torch.empty_like(q, device=DEV)
+    gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, window)
+    want = torch.empty_like(q)
+    PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, window)
+    close(out, want, dtype, scale=1.0 if dtype == torch.float32 else 2.0)
+
+
+@pytest.mark.parametrize("parts", [1, 2, 7, 64])
+@pytest.mark.parametrize("window", [None, 300])
+def test_decode_split_over_waves(parts, window):
+    """The decode kernel with its keys split over any number of waves, merged by the second kernel."""
+    q_lens = [1, 1, 1, 1, 1]
+    ctx_lens = [1, 15, 16, 700, 1025]
+    q, kc, vc, meta = _attention_case(torch.bfloat16, 8, 2, 128, 16, window, q_lens, ctx_lens, seed=3)
+    out = torch.empty_like(q, device=DEV)
+    gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), 128 ** -0.5, window, parts=parts)
+    want = torch.empty_like(q)
+    PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), 128 ** -0.5, window)
+    close(out, want, torch.bfloat16, scale=2.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_far_key_among_hundreds(dtype):
+    """One key far back carries nearly all the weight: an attention that drops or misplaces it
+    (a wrong page, a partition edge, a tile edge) gives a visibly different output."""
+    for key in (0, 15, 16, 255, 256, 511):
+        q, kc, vc, meta = _attention_case(dtype, 8, 2, 64, 16, None, [40, 1], [700, 600], seed=key,
+                                          scale_one=(1, key, 3.0))
+        q2, kc2, vc2, meta2 = _attention_case(dtype, 8, 2, 64, 16, None, [40, 1], [700, 600], seed=key,
+                                              scale_one=(0, key, 3.0))
+        for (qq, kk, vv, mm) in ((q, kc, vc, meta), (q2, kc2, vc2, meta2)):
+            out = torch.empty_like(qq, device=DEV)
+            gpu_ops().paged_attention(qq.to(DEV), kk.to(DEV), vv.to(DEV), out, mm(DEV), 64 ** -0.5, None)
+            want = torch.empty_like(qq)
+            PLAIN.paged_attention(qq, kk, vv, want, mm("cpu"), 64 ** -0.5, None)
+            close(out, want, dtype, scale=1.0 if dtype == torch.float32 else 2.0)
+
+
+def test_window_edge():
+    """Keys exactly at the window's edge: position p - W + 1 is seen, p - W is not."""
+    w = 40
+    for dtype in DTYPES:
+        for ctx in (w - 1, w, w + 1, 2 * w, 129):
+            for boost_key in (ctx - w, ctx - w - 1):
+                if boost_key < 0:
+                    continue
+                q, kc, vc, meta = _attention_case(dtype, 4, 2, 64, 16, w, [1], [ctx], seed=ctx, scale_one=(0, boost_key, 3.0))
+                out = torch.empty_like(q, device=DEV)
+                gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), 0.125, w)
+                want = torch.empty_like(q)
+                PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), 0.125, w)
+                close(out, want, dtype, scale=1.0 if dtype == torch.float32 else 2.0)
+
+
+# ------------------------------------------------------------------ sampling
+
+
+def test_sample_greedy_and_ties():
+    logits = rnd((9, 517), torch.float32, 30)
+    logits[3, 100] = logits[3, 400] = 50.0   # a tie: the lower index wins
+    out = torch.empty(9, dtype=torch.int32, device=DEV)
+    gpu_ops().sample(logits.to(DEV), None, out)
+    want = logits.argmax(dim=-1)
+    want[3] = 100
+    assert out.cpu().tolist() == want.tolist()
+
+
+def test_noise_is_the_stated_mix():
+    seeds = torch.tensor([0, 7, 2 ** 40 + 3], dtype=torch.int64)
+    counters = torch.tensor([0, 5, 123456], dtype=torch.int64)
+    got = gpu_ops().exponential_noise(seeds.to(DEV), counters.to(DEV), 311).cpu()
+    want = torch.stack([exponential_noise_row(int(s), int(c), 311) for s, c in zip(seeds, counters)])
+    assert torch.allclose(got, want, rtol=2e-6, atol=1e-7)
+    big = gpu_ops().exponential_noise(torch.arange(64, dtype=torch.int64, device=DEV),
+                                      torch.zeros(64, dtype=torch.int64, device=DEV), 4096)
+    assert abs(float(big.mean()) - 1.0) < 0.01 and abs(float(big.var()) - 1.0) < 0.03
+
+
+@pytest.mark.parametrize("top_k,top_p", [(-1, 1.0), (5, 1.0), (-1, 0.6), (20, 0.9), (1, 1.0)])
+def test_sample_matches_plain_given_noise(top_k, top_p):
+    rows, vocab = 12, 311
+    logits = rnd((rows, vocab), torch.float32, 31, 2.0)
+    temps = torch.tensor([0.7, 1.0, 0.0, 1.3] * 3, dtype=torch.float32)
+    noise = torch.empty((rows, vocab)).exponential_(generator=torch.Generator().manual_seed(32))
+    ks = torch.full((rows,), top_k, dtype=torch.int32)
+    ps = torch.full((rows,), top_p, dtype=torch.float32)
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    gpu_ops().sample(logits.to(DEV), temps.to(DEV), out, top_ks=ks.to(DEV), top_ps=ps.to(DEV), noise=noise.to(DEV))
+    want = torch.empty(rows, dtype=torch.int32)
+    PLAIN.sample(logits, temps, want, top_ks=ks, top_ps=ps, noise=noise)
+    assert out.cpu().tolist() == want.tolist()
+    if top_k == 1:
+        assert out.cpu().tolist() == logits.argmax(dim=-1).tolist()
+
+
+def test_sample_frequencies_follow_softmax():
+    vocab, draws = 11, 20000
+    logits = torch.tensor([[2.0, 1.0, 0.5, 0.0, -1.0, 1.5, 0.2, -3.0, 0.9, 1.1, -0.5]])
+    temp = 0.7
+    rep = logits.repeat(draws, 1).to(DEV)
+    out = torch.empty(draws, dtype=torch.int32, device=DEV)
+    gpu_ops().sample(rep, torch.full((draws,), temp, device=DEV), out,
+                     seeds=torch.full((draws,), 1234, dtype=torch.int64, device=DEV),
+                     counters=torch.arange(draws, dtype=torch.int64, device=DEV))
+    freq = torch.bincount(out.cpu().long(), minlength=vocab).double() / draws
+    want = torch.softmax(logits[0].double() / temp, dim=-1)
+    assert float((freq - want).abs().max()) < 4 * math.sqrt(0.25 / draws)
+
+
+def test_sample_does_not_depend_on_batch():
+    logits = rnd((6, 517), torch.float32, 33, 2.0).to(DEV)
+    temps = torch.full((6,), 0.8, device=DEV)
+    seeds = torch.tensor([5, 6, 7, 8, 9, 10], dtype=torch.int64, device=DEV)
+    counters = torch.tensor([0, 3, 1, 4, 1, 5], dtype=torch.int64, device=DEV)
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    gpu_ops().sample(logits, temps, out, seeds=seeds, counters=counters)
+    for r in (0, 2, 5):
+        one = torch.empty(1, dtype=torch.int32, device=DEV)
+        gpu_ops().sample(logits[r:r + 1].contiguous(), temps[r:r + 1].contiguous(), one,
+                         seeds=seeds[r:r + 1].contiguous(), counters=counters[r:r + 1].contiguous())
+        assert int(one) == int(out[r])
+
+
+def test_kernels_refuse_what_they_cannot_take():
+    ops = gpu_ops()
+    x = torch.zeros((4, 64), device=DEV)
+    with pytest.raises(KernelError):
+        ops.rmsnorm(x, torch.ones(63, device=DEV), 1e-6, torch.empty_like(x))
+    with pytest.raises(KernelError):
+        ops.rmsnorm(x.cpu(), torch.ones(64), 1e-6, torch.empty_like(x.cpu()))
+    with pytest.raises(KernelError):
+        ops.rmsnorm(torch.zeros((2, 20000), device=DEV), torch.ones(20000, device=DEV), 1e-6,
+                    torch.zeros((2, 20000), device=DEV))
+    with pytest.raises(KernelError):
+        ops.silu_mul(torch.zeros((2, 7), device=DEV), torch.zeros((2, 3), device=DEV))
+    with pytest.raises(KernelError):
+        ops.linear(x, torch.zeros((5, 63), device=DEV))
+    with pytest.raises(KernelError):
+        ops.embedding(torch.zeros((10, 8), device=DEV, dtype=torch.float16), torch.zeros(2, dtype=torch.int32, device=DEV),
+                      torch.zeros((2, 8), device=DEV))
