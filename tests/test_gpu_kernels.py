@@ -221,7 +221,7 @@ def test_paged_attention_mixed_batch(dtype, hq, hkv, d, page, window):
     gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, window)
     want = torch.empty_like(q)
     PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, window)
-    close(out, want, dtype, scale=1.0 if dtype == torch.float32 else 2.0)
+    close(out, want, dtype)
 
 
 @pytest.mark.parametrize("parts", [1, 2, 7, 64])
@@ -235,7 +235,7 @@ def test_decode_split_over_waves(parts, window):
     gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), 128 ** -0.5, window, parts=parts)
     want = torch.empty_like(q)
     PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), 128 ** -0.5, window)
-    close(out, want, torch.bfloat16, scale=2.0)
+    close(out, want, torch.bfloat16)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -252,7 +252,7 @@ def test_far_key_among_hundreds(dtype):
             gpu_ops().paged_attention(qq.to(DEV), kk.to(DEV), vv.to(DEV), out, mm(DEV), 64 ** -0.5, None)
             want = torch.empty_like(qq)
             PLAIN.paged_attention(qq, kk, vv, want, mm("cpu"), 64 ** -0.5, None)
-            close(out, want, dtype, scale=1.0 if dtype == torch.float32 else 2.0)
+            close(out, want, dtype)
 
 
 def test_window_edge():
@@ -268,7 +268,7 @@ def test_window_edge():
                 gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), 0.125, w)
                 want = torch.empty_like(q)
                 PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), 0.125, w)
-                close(out, want, dtype, scale=1.0 if dtype == torch.float32 else 2.0)
+                close(out, want, dtype)
 
 
 # ------------------------------------------------------------------ sampling
