@@ -55,8 +55,8 @@ class Config:
         if self.max_model_len is None:
             self.max_model_len = mc.max_position_embeddings
         self.max_model_len = min(self.max_model_len, mc.max_position_embeddings)
-        if self.kv_cache_block_size <= 0 or self.kv_cache_block_size % 8:
-            raise ConfigError("kv_cache_block_size must be a positive multiple of 8")
+        if self.kv_cache_block_size <= 0 or self.kv_cache_block_size % 4:
+            raise ConfigError("kv_cache_block_size must be a positive multiple of 4")
         # atom/config.py:1755-1767
         if self.long_prefill_token_threshold:
             if self.long_prefill_token_threshold > self.max_model_len:

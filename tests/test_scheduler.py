@@ -1,0 +1,275 @@
+"""The scheduler's decisions, on token lists alone (no model): admission, the token
+budget and how prompts are cut, mixed batches, what happens when pages run out, and the
+finishing rules.  Vectors marked (ref) are the reference's own
+(tests/test_scheduler.py in ROCm/ATOM)."""
+
+import pytest
+
+from atom_amd.cache import CacheManager, GroupSpec
+from atom_amd.config import Config, model_config_from_dict
+from atom_amd.engine.scheduler import Scheduler
+from atom_amd.engine.sequence import Sequence, SequenceStatus
+from atom_amd.sampling import SamplingParams
+from tiny import TINY_C
+
+
+class FakeCore:
+    """What the scheduler needs of the engine core: the cache manager and open/close."""
+
+    def __init__(self, groups, slots):
+        self.manager = CacheManager(groups, slots)
+
+    def open(self, rid):
+        if rid not in self.manager:
+            self.manager.open(rid)
+
+    def close(self, rid):
+        if rid in self.manager:
+            self.manager.close(rid)
+
+
+def make(blocks=100, block=4, window_group=None, **kw):
+    raw = {**TINY_C, "max_position_embeddings": 4096, "eos_token_id": 2}
+    kw.setdefault("max_num_seqs", 4)
+    kw.setdefault("max_num_batched_tokens", 64)
+    kw.setdefault("max_model_len", 1024)
+    cfg = Config("x", model_config=model_config_from_dict(raw), kv_cache_block_size=block, **kw)
+    groups = [GroupSpec(block, blocks)]
+    if window_group:
+        groups.append(GroupSpec(block, window_group[1], window=window_group[0]))
+    core = FakeCore(groups, cfg.max_num_seqs)
+    return Scheduler(cfg, core), core
+
+
+def seq(tokens, **sp):
+    return Sequence(list(tokens), SamplingParams(**sp))
+
+
+def run(sched, batch, token=5):
+    """Pretends the step ran: every final item samples ``token``."""
+    sampled = {it.seq.id: (token(it.seq) if callable(token) else token) for it in batch.items if it.is_final}
+    return sched.postprocess(batch, sampled)
+
+
+def test_budget_two_prompts_128_64():   # (ref) :236-254
+    sched, _ = make(max_num_batched_tokens=192, blocks=100)
+    sched.add(seq(range(128)))
+    sched.add(seq(range(200, 328)))
+    batch = sched.schedule()
+    assert [it.num_tokens for it in batch.items] == [128, 64]
+    assert [it.is_final for it in batch.items] == [True, False]
+
+
+def test_budget_sliver_is_left_for_the_next_step():   # (ref) :256-278
+    sched, _ = make(max_num_batched_tokens=200, blocks=400)
+    for start in (0, 200, 400):
+        sched.add(seq(range(start, start + 128)))
+    batch = sched.schedule()
+    assert [it.num_tokens for it in batch.items] == [128, 64]     # 8 tokens stay unspent
+    assert len(sched.waiting) == 1
+
+
+def test_prompt_cut_6_then_4():   # (ref) :280-314
+    sched, _ = make(max_num_batched_tokens=6, blocks=100, block=4)
+    s = seq(range(10))
+    sched.add(s)
+    b1 = sched.schedule()
+    assert b1.entries()[0].tokens == list(range(6)) and b1.items[0].start == 0
+    assert b1.entries()[0].want == []
+    run(sched, b1)
+    assert s.is_partial_prefill and s.num_cached_tokens == 6 and s.num_completion_tokens == 0
+    b2 = sched.schedule()
+    assert b2.entries()[0].tokens == list(range(6, 10)) and b2.items[0].start == 6
+    assert b2.entries()[0].want == [3]
+    run(sched, b2)
+    assert not s.is_partial_prefill and s.num_cached_tokens == 10 and s.token_ids[-1] == 5
+
+
+def test_chunking_off_is_all_or_nothing():
+    sched, _ = make(max_num_batched_tokens=12, enable_chunked_prefill=False)
+    sched.add(seq(range(8)))
+    sched.add(seq(range(8)))
+    assert [it.num_tokens for it in sched.schedule().items] == [8]
+    sched2, _ = make(max_num_batched_tokens=12, enable_chunked_prefill=False)
+    s = seq(range(20))
+    sched2.add(s)
+    assert sched2.schedule() is None
+    assert sched2.take_rejected() == [s] and s.leave_reason.startswith("unschedulable")
+
+
+def test_admission_respects_pages_and_blocks_the_queue():   # (ref) :316-321
+    sched, _ = make(blocks=1, block=4)
+    sched.add(seq([1, 2, 3, 4]))
+    sched.add(seq([5, 6, 7, 8, 9]))     # two pages: can never run in a pool of one
+    sched.add(seq([1, 2]))
+    batch = sched.schedule()
+    assert [it.num_tokens for it in batch.items] == [4]
+    rejected = sched.take_rejected()
+    assert len(rejected) == 1 and "cache pages" in rejected[0].leave_reason
+    assert len(sched.waiting) == 1      # the short one waits behind: pages are taken
+
+
+def test_too_long_prompt_is_rejected_not_hung():
+    sched, _ = make(max_model_len=16)
+    s = seq(range(17))
+    sched.add(s)
+    assert sched.schedule() is None
+    assert sched.take_rejected() == [s] and "max_model_len" in s.leave_reason and s.is_finished
+    assert sched.is_finished()
+
+
+def test_max_num_seqs():
+    sched, _ = make(max_num_seqs=2)
+    for _ in range(3):
+        sched.add(seq(range(4)))
+    assert len(sched.schedule().items) == 2
+    assert len(sched.waiting) == 1
+
+
+def test_decode_and_prompt_share_one_step():
+    sched, _ = make(max_num_batched_tokens=70)
+    a = seq(range(8), max_tokens=10)
+    sched.add(a)
+    run(sched, sched.schedule())
+    b = seq(range(100, 200), max_tokens=10)
+    sched.add(b)
+    batch = sched.schedule()
+    kinds = [(it.seq.id, it.is_decode, it.num_tokens) for it in batch.items]
+    # the decode token first; of the 69 tokens left the prompt gets 64 (a cut portion is floored to 64s)
+    assert kinds == [(a.id, True, 1), (b.id, False, 64)]
+    assert batch.entries()[0].tokens == [5] and batch.entries()[0].want == [0]
+    assert batch.entries()[1].want == []
+    run(sched, batch)
+    batch = sched.schedule()
+    assert [(it.is_decode, it.num_tokens, it.is_final) for it in batch.items] == [(True, 1, True), (False, 36, True)]
+    run(sched, batch)
+    batch = sched.schedule()
+    assert [(it.is_decode, it.num_tokens) for it in batch.items] == [(True, 1), (True, 1)]
+
+
+def test_decode_preemption():   # (ref) :332-346
+    sched, core = make(blocks=2, block=4)
+    s1, s2 = seq([1, 2, 3, 4], max_tokens=8), seq([5, 6, 7, 8], max_tokens=8)
+    sched.add(s1)
+    sched.add(s2)
+    run(sched, sched.schedule(), token=9)
+    batch = sched.schedule()
+    assert {s1.status, s2.status} == {SequenceStatus.RUNNING, SequenceStatus.WAITING}
+    assert s2.status == SequenceStatus.WAITING, "the last running request is the one preempted"
+    assert [it.seq.id for it in batch.items] == [s1.id] and sched.total_preemptions == 1
+    assert s2.num_cached_tokens == 0 and s2.id not in core.manager
+    assert sched.waiting[0] is s2
+    core.manager.check()
+
+
+def test_preempted_request_prefills_prompt_plus_generated():
+    sched, core = make(blocks=3, block=4, max_num_batched_tokens=64)
+    s1, s2 = seq([1, 2, 3, 4], max_tokens=3), seq([5, 6, 7, 8], max_tokens=6)
+    sched.add(s1)
+    sched.add(s2)
+    run(sched, sched.schedule(), token=9)        # both prompts; 2 pages held, 1 free
+    run(sched, sched.schedule(), token=9)        # s1 takes the last page; s2 cannot: preempted
+    assert s2.status == SequenceStatus.WAITING and s2.token_ids == [5, 6, 7, 8, 9]
+    run(sched, sched.schedule(), token=9)        # s1 decodes (pool still full for s2)
+    assert s1.is_finished and s1.leave_reason == "max_tokens"
+    batch = sched.schedule()
+    assert [it.seq.id for it in batch.items] == [s2.id]
+    assert batch.entries()[0].tokens == [5, 6, 7, 8, 9] and not batch.items[0].is_decode
+    assert batch.entries()[0].want == [4]
+    run(sched, batch, token=9)
+    assert s2.token_ids == [5, 6, 7, 8, 9, 9] and s2.num_cached_tokens == 5
+    core.manager.check()
+
+
+def test_lone_request_that_outgrows_the_pool_preempts_itself_then_is_rejected():
+    sched, core = make(blocks=1, block=4)
+    s = seq([1, 2, 3], max_tokens=10)
+    sched.add(s)
+    run(sched, sched.schedule())
+    run(sched, sched.schedule())          # 4 tokens cached + 1 pending: needs a second page
+    assert sched.schedule() is None       # preempted itself; now 5 tokens need 2 pages of a pool of 1
+    out = sched.take_rejected()
+    assert out == [s] and "cache pages" in s.leave_reason
+    assert core.manager.num_free_pages() == 1 and sched.is_finished()
+
+
+@pytest.mark.parametrize("kw,tokens,reason,count", [
+    (dict(max_tokens=3), [7, 7, 7, 7], "max_tokens", 3),
+    (dict(max_tokens=9), [7, 2, 7], "eos", 2),
+    (dict(max_tokens=4, ignore_eos=True), [2, 2, 2, 2, 2], "max_tokens", 4),
+])
+def test_finish_reasons(kw, tokens, reason, count):   # (ref) :1110-1177
+    sched, core = make()
+    s = seq([1, 1, 1], **kw)
+    sched.add(s)
+    feed = iter(tokens)
+    while not s.is_finished:
+        run(sched, sched.schedule(), token=lambda _s: next(feed))
+    assert s.leave_reason == reason and s.num_completion_tokens == count
+    assert not sched.running and s.id not in core.manager
+
+
+def test_stop_token_ids_and_stop_sequences():
+    sched, _ = make()
+    sched.stop_token_ids = {11}
+    s = seq([1, 1], max_tokens=9)
+    sched.add(s)
+    feed = iter([7, 11])
+    while not s.is_finished:
+        run(sched, sched.schedule(), token=lambda _s: next(feed))
+    assert s.leave_reason == "stop_11"
+    s2 = Sequence([1, 1], SamplingParams(max_tokens=9), stop_token_sequences=[[8, 9]])
+    sched.add(s2)
+    feed = iter([8, 8, 9, 3])
+    while not s2.is_finished:
+        run(sched, sched.schedule(), token=lambda _s: next(feed))
+    assert s2.leave_reason == "stop_sequence" and s2.completion_token_ids == [8, 8, 9]
+    # a stop sequence wins over eos when both end at the same token
+    s3 = Sequence([1], SamplingParams(max_tokens=9), stop_token_sequences=[[4, 2]])
+    sched.add(s3)
+    feed = iter([4, 2])
+    while not s3.is_finished:
+        run(sched, sched.schedule(), token=lambda _s: next(feed))
+    assert s3.leave_reason == "stop_sequence"
+
+
+def test_sequence_stops_at_max_model_len():
+    sched, _ = make(max_model_len=6)
+    s = seq([1, 1, 1, 1], max_tokens=50)
+    sched.add(s)
+    while not s.is_finished:
+        run(sched, sched.schedule())
+    assert s.leave_reason == "max_model_len" and s.num_tokens == 6
+
+
+def test_long_prefill_threshold_caps_a_portion():
+    sched, _ = make(max_num_batched_tokens=512, long_prefill_token_threshold=64, blocks=400)
+    s = seq(range(200))
+    sched.add(s)
+    sizes = []
+    while s.num_completion_tokens == 0:
+        batch = sched.schedule()
+        sizes.append(batch.items[0].num_tokens)
+        run(sched, batch)
+    assert sizes == [64, 64, 64, 8]
+
+
+def test_whole_prompt_is_reserved_at_admission_where_all_keys_are_kept():
+    sched, core = make(blocks=6, block=4, max_num_batched_tokens=8, window_group=(8, 20))
+    a = seq(range(20))
+    sched.add(a)
+    sched.add(seq(range(8)))
+    batch = sched.schedule()
+    assert [it.num_tokens for it in batch.items] == [8]
+    assert len(core.manager.block_table(a.id, 0)) == 5, "all five pages of the prompt are held from the start"
+    assert len(core.manager.block_table(a.id, 1)) == 2, "the window group holds this step only"
+    assert len(sched.waiting) == 1, "the second prompt waits: one free page is not enough for it"
+
+
+def test_aborted_waiting_request_leaves_without_running():
+    sched, _ = make()
+    s = seq(range(4))
+    s.status = SequenceStatus.ABORTED
+    sched.add(s)
+    assert sched.schedule() is None
+    assert sched.take_rejected() == [s] and s.leave_reason == "aborted"
