@@ -1,0 +1,140 @@
+"""Generation through the entry points on the GPU: greedy against the plain implementation,
+long decoding, the first tokens of a sequence, seeded temperature sampling that does not
+depend on the batch, page pressure with preemption, and the command line."""
+
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_model as pm
+from helpers import gpu_ops, oracle_weights, random_ids, tiny_folder
+from tiny import CONFIGS, PAGE
+from atom_amd import LLMEngine, SamplingParams
+from replay import ROOT
+
+pytestmark = pytest.mark.gpu
+
+
+def engine(which, dtype, **kw):
+    kw.setdefault("kv_cache_block_size", PAGE[which])
+    kw.setdefault("num_kvcache_blocks", 64)
+    kw.setdefault("max_num_seqs", 4)
+    return LLMEngine(tiny_folder(which), dtype=dtype, ops=gpu_ops(), **kw)
+
+
+def check_greedy(which, dtype, prompts, outs):
+    """Every generated token is the plain implementation's argmax, or, in bfloat16, a token whose
+    plain logit is within rounding of the best."""
+    cfg, tensors = oracle_weights(which)
+    for prompt, out in zip(prompts, outs):
+        ids = list(prompt)
+        for step, token in enumerate(out["token_ids"]):
+            logits = pm.qwen3_logits(cfg, tensors, ids)[-1]
+            best = int(logits.argmax())
+            slack = 0.0 if dtype == "fp32" else 0.03 * float(logits.abs().max())
+            assert token == best or float(logits[best] - logits[token]) <= slack, \
+                f"{which}/{dtype}: token {step} of a {len(prompt)}-token prompt is {token}, plain says {best}"
+            ids.append(token)
+
+
+@pytest.mark.parametrize("which,dtype", [("A", "fp32"), ("B", "fp32"), ("B", "bf16"), ("C", "fp32"), ("C", "bf16")])
+def test_greedy_generation_matches_plain(which, dtype):
+    lens = {"A": (5, 17, 33), "B": (1, 9, 40, 71), "C": (3, 50, 120)}[which]
+    prompts = [random_ids(which, n, 40 + n) for n in lens]
+    llm = engine(which, dtype, max_num_batched_tokens=16 if which == "B" else 64)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8 if which == "A" else 12, ignore_eos=True))
+    assert [o["num_tokens_input"] for o in outs] == list(lens)
+    assert all(o["finish_reason"] == "max_tokens" and o["ttft"] > 0 and o["latency"] >= o["ttft"] for o in outs)
+    check_greedy(which, dtype, prompts, outs)
+    llm.core.manager.check()
+    assert all(p.num_free == p.num_pages for p in llm.core.manager.pools)
+
+
+def test_long_decoding_past_the_window_and_many_pages():
+    """200 decoded tokens in float32: every token is the plain argmax; the window layers' pages go back meanwhile."""
+    prompt = random_ids("C", 30, 7)
+    llm = engine("C", "fp32", num_kvcache_blocks=20)
+    out = llm.generate([prompt], SamplingParams(temperature=0.0, max_tokens=200, ignore_eos=True))[0]
+    assert out["num_tokens_output"] == 200
+    check_greedy("C", "fp32", [prompt], [out])
+
+
+def test_first_tokens_of_a_sequence():
+    """Prompts of one and two tokens: the first position has a single key, itself."""
+    for which in ("A", "B"):
+        for dtype in ("fp32", "bf16"):
+            prompts = [[3], [7, 250 % CONFIGS[which]["vocab_size"]], [0]]
+            outs = engine(which, dtype).generate(prompts, SamplingParams(temperature=0.0, max_tokens=3, ignore_eos=True))
+            check_greedy(which, dtype, prompts, outs)
+
+
+def test_seeded_temperature_sampling_is_reproducible_and_batch_independent():
+    prompts = [random_ids("B", n, 60 + n) for n in (9, 40, 71)]
+    sp = [SamplingParams(temperature=0.7, max_tokens=12, ignore_eos=True, seed=100 + k) for k in range(3)]
+    together = engine("B", "fp32", max_num_batched_tokens=16).generate(prompts, sp)
+    again = engine("B", "fp32", max_num_batched_tokens=64).generate(prompts, sp)
+    assert [o["token_ids"] for o in together] == [o["token_ids"] for o in again]
+    alone = engine("B", "fp32").generate([prompts[1]], sp[1])[0]
+    assert alone["token_ids"] == together[1]["token_ids"], "a request's draws do not depend on its batch-mates"
+    other = engine("B", "fp32").generate([prompts[1]], SamplingParams(temperature=0.7, max_tokens=12, ignore_eos=True, seed=999))[0]
+    assert other["token_ids"] != alone["token_ids"]
+    greedy = engine("B", "fp32").generate([prompts[1]], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))[0]
+    topk1 = engine("B", "fp32").generate([prompts[1]], SamplingParams(temperature=0.7, top_k=1, max_tokens=12, ignore_eos=True))[0]
+    assert topk1["token_ids"] == greedy["token_ids"], "top_k = 1 is greedy"
+
+
+def test_sampled_tokens_follow_the_plain_race():
+    """With the engine's own noise fed to the plain race, every sampled token is reproduced."""
+    from plain_kernels import exponential_noise_row
+    cfg, tensors = oracle_weights("B")
+    prompt = random_ids("B", 20, 5)
+    out = engine("B", "fp32").generate([prompt], SamplingParams(temperature=0.7, max_tokens=6, ignore_eos=True, seed=42))[0]
+    ids = list(prompt)
+    for k, token in enumerate(out["token_ids"]):
+        logits = pm.qwen3_logits(cfg, tensors, ids)[-1:]
+        noise = exponential_noise_row(42, k, cfg["vocab_size"]).unsqueeze(0)
+        assert int(pm.exponential_race(logits, torch.tensor([0.7]), noise)[0]) == token
+        ids.append(token)
+
+
+def test_page_pressure_preempts_and_still_matches():
+    """Six requests through a pool that cannot hold them all: some are preempted, prefilled again with
+    what they had generated, and still produce the plain implementation's tokens."""
+    prompts = [random_ids("B", n, 80 + n) for n in (30, 25, 41, 12, 36, 19)]
+    llm = engine("B", "fp32", num_kvcache_blocks=14, max_num_seqs=4, max_num_batched_tokens=64)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True))
+    assert llm.scheduler.total_preemptions > 0, "the pool was meant to be too small"
+    assert all(o["finish_reason"] == "max_tokens" and o["num_tokens_output"] == 20 for o in outs)
+    check_greedy("B", "fp32", prompts, outs)
+    llm.core.manager.check()
+
+
+def test_stop_on_eos_and_logprobs():
+    cfg, tensors = oracle_weights("B")
+    prompt = random_ids("B", 9, 3)
+    free = engine("B", "fp32").generate([prompt], SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True, logprobs=True))[0]
+    eos = free["token_ids"][3]
+    first = free["token_ids"].index(eos)
+    llm = engine("B", "fp32", eos_token_id=eos)
+    out = llm.generate([prompt], SamplingParams(temperature=0.0, max_tokens=10))[0]
+    assert out["finish_reason"] == "eos" and out["token_ids"] == free["token_ids"][:first + 1]
+    lp = torch.log_softmax(pm.qwen3_logits(cfg, tensors, prompt)[-1], dim=-1)[free["token_ids"][0]]
+    assert abs(free["logprobs"][0] - float(lp)) < 1e-4
+    rejected = llm.generate([list(range(300))], SamplingParams(max_tokens=2))[0]
+    assert rejected["finish_reason"].startswith("unschedulable")
+
+
+def test_command_line():
+    cmd = [sys.executable, "-m", "atom_amd.examples.simple_inference", "--model", tiny_folder("A"), "--temperature", "0",
+           "--max-tokens", "8", "--block_size", "16", "--num-kvcache-blocks", "32", "--max-num-seqs", "4", "--dtype", "fp32",
+           "--seed", "3"]
+    res = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert res.stdout.count("Completion:") == 3 and res.stdout.count("finish_reason=max_tokens") == 3
+    import random, re
+    rng = random.Random(3)
+    prompts = [[rng.randrange(256) for _ in range(n)] for n in (5, 17, 33)]
+    shown = [eval(m) for m in re.findall(r"Completion: (\[.*?\])", res.stdout)]
+    check_greedy("A", "fp32", prompts, [{"token_ids": ids} for ids in shown])

@@ -1,0 +1,342 @@
+"""Each part alone on the GPU against the plain implementation's function of the same
+name, in float32 and bfloat16; and a toy mixer with a state of its own, defined here,
+registered, built into a model through the registries and stepped through the engine
+without a change to the framework's files."""
+
+from dataclasses import dataclass
+from typing import ClassVar
+
+import pytest
+import torch
+
+import plain_model as pm
+from helpers import gpu_ops
+from atom_amd.cache import CacheManager, GroupSpec
+from atom_amd.config import ModelConfig, register_architecture, unregister_architecture
+from atom_amd.engine.context import KVBinding, StepContext
+from atom_amd.engine.core import StepEntry, build_core, load_model
+from atom_amd.kernels.hip import AttentionMeta
+from atom_amd.models.model import ModelSpec
+from atom_amd.parts import (FEED_FORWARDS, MIXERS, NORMS, GatedMLP, GroupedQueryAttention, LMHead, Mixer, ParamSpec,
+                            PartChoice, PreNormBlock, RMSNorm, RotaryEncoding, StateNeed, TokenEmbedding)
+from atom_amd.weights import write_random_model
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2.5e-2}
+
+
+def rnd(shape, seed, scale=1.0):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def fill(part, dtype, seed=0, scale=0.3):
+    """Random parameters for a part and its children; returns them by full name in float64."""
+    out = {}
+    for k, p in enumerate(part.walk()):
+        for local, spec in p.param_specs().items():
+            value = rnd(spec.shape, seed * 1000 + k * 10 + len(out), scale)
+            if spec.init == "one_plus_normal":
+                value = 1 + value
+            target = torch.float32 if spec.kind == "vector" else dtype
+            p.params[local] = value.to(target).to(DEV)
+            out[p.full_name(local)] = p.params[local].double().cpu()
+        p.finalize(torch.device(DEV), dtype)
+    return out
+
+
+def ctx_for(dtype, positions, page_size=16, group=0, num_pages=None):
+    """A one-request step context: the request's tokens at ``positions`` (consecutive)."""
+    n = len(positions)
+    end = positions[-1] + 1
+    num_pages = num_pages or -(-end // page_size) + 2
+    mgr = CacheManager([GroupSpec(page_size, num_pages)], 1)
+    mgr.open("r")
+    mgr.cover("r", 0, end)
+    table = torch.tensor([mgr.block_table("r", 0)], dtype=torch.int32, device=DEV)
+    pos = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    meta = AttentionMeta(
+        token_seq=torch.zeros(n, dtype=torch.int32, device=DEV), positions=pos, block_tables=table,
+        cu_seqlens_q=torch.tensor([0, n], dtype=torch.int32, device=DEV),
+        context_lens=torch.tensor([end], dtype=torch.int32, device=DEV), num_seqs=1, num_tokens=n, max_q_len=n,
+        max_context_len=end, page_size=page_size, num_prefill=1 if n > 1 else 0,
+        prefill_tiles=torch.tensor([(0, r) for r in range(0, n, 32)], dtype=torch.int32, device=DEV) if n > 1 else None,
+        rows_per_tile=32)
+    slots = torch.from_numpy(mgr.slot_mapping("r", 0, positions[0], n)).to(DEV)
+    return StepContext(ops=gpu_ops(), dtype=dtype, device=torch.device(DEV), num_tokens=n, num_seqs=1, positions=pos,
+                       attention={group: meta}, slot_mappings={group: slots}, seq_starts=[0], seq_lens=[n],
+                       seq_cached=[positions[0]], state_slots=[0]), num_pages
+
+
+def check(got, want, dtype):
+    got, want = got.double().cpu(), want.double()
+    scale = max(1e-6, float(want.abs().max()))
+    assert float((got - want).abs().max()) <= TOL[dtype] * scale
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_part(dtype):
+    norm = RMSNorm(136, 3e-6, prefix="n")
+    w = fill(norm, dtype)["n.weight"]
+    ctx, _ = ctx_for(dtype, [0, 1, 2, 3, 4])
+    x = rnd((5, 136), 1, 2.0).to(dtype)
+    check(norm.forward(ctx, x.to(DEV)), pm.rms_norm(x.double(), w, 3e-6), dtype)
+    y, res = norm.forward_residual(ctx, x.to(DEV), None)
+    assert res.dtype == torch.float32 and torch.equal(res.cpu(), x.float())
+    check(y, pm.rms_norm(x.double(), w, 3e-6), dtype)
+    x2 = rnd((5, 136), 2).to(dtype)
+    y2, res2 = norm.forward_residual(ctx, x2.to(DEV), res)
+    want_y, want_res = pm.add_rms_norm(x2.double(), x.double(), w, 3e-6)
+    check(y2, want_y, dtype)
+    check(res2, want_res, torch.float32)
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    y3 = norm.forward_rows(ctx, x2.to(DEV), res2.clone(), rows)
+    want3, _ = pm.add_rms_norm(x2.double()[[4, 1]], res2.double().cpu()[[4, 1]], w, 3e-6)
+    check(y3, want3, dtype)
+
+
+def test_rotary_tables():
+    rope = RotaryEncoding(head_dim=64, theta=5e5, max_positions=300)
+    rope.finalize(torch.device(DEV), torch.bfloat16)
+    cos, sin = pm.rope_angles(torch.arange(300), 64, 5e5)
+    assert rope.cos.dtype == torch.float32 and rope.cos.shape == (300, 32)
+    assert torch.equal(rope.cos.cpu(), cos) and torch.equal(rope.sin.cpu(), sin)
+    with pytest.raises(ValueError):
+        RotaryEncoding(head_dim=64, theta=1e4, max_positions=8, rotary_dim=65)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,d,bias,window", [(4, 2, 16, False, None), (6, 3, 32, True, None), (8, 2, 64, True, 9),
+                                                  (3, 3, 48, False, None)])
+def test_attention_part(dtype, hq, hkv, d, bias, window):
+    hidden = 72
+    rope = PartChoice("rotary", {"theta": 1e4, "max_positions": 128})
+    attn = GroupedQueryAttention(hidden, hq, hkv, d, qkv_bias=bias, qk_norm=True, norm_eps=1e-5, window=window,
+                                 position_encoding=rope, prefix="a")
+    w = fill(attn, dtype, seed=3, scale=0.2)
+    n = 37
+    ctx, pages = ctx_for(dtype, list(range(n)), page_size=8)
+    cache = KVBinding(0, torch.zeros((pages, hkv, 8, d), dtype=dtype, device=DEV),
+                      torch.zeros((pages, hkv, d, 8), dtype=dtype, device=DEV))
+    x = rnd((n, hidden), 4).to(dtype)
+    got = attn.forward(ctx, x.to(DEV), cache)
+    qkv = w["a.qkv.weight"]
+    plain_w = {"q_proj.weight": qkv[:hq * d], "k_proj.weight": qkv[hq * d:(hq + hkv) * d],
+               "v_proj.weight": qkv[(hq + hkv) * d:], "o_proj.weight": w["a.o.weight"],
+               "q_norm.weight": w["a.q_norm.weight"], "k_norm.weight": w["a.k_norm.weight"]}
+    if bias:
+        b = w["a.qkv.bias"]
+        plain_w.update({"q_proj.bias": b[:hq * d], "k_proj.bias": b[hq * d:(hq + hkv) * d], "v_proj.bias": b[(hq + hkv) * d:]})
+    cfg = dict(num_attention_heads=hq, num_key_value_heads=hkv, head_dim=d, rms_norm_eps=1e-5, rope_theta=1e4)
+    want, _ = pm.self_attention(x.double(), torch.arange(n), plain_w, cfg, window)
+    check(got, want, dtype)
+    # the same tokens in two steps over the cache the first step left
+    cache2 = KVBinding(0, torch.zeros_like(cache.k_cache), torch.zeros_like(cache.v_cache))
+    ctx_a, _ = ctx_for(dtype, list(range(20)), page_size=8, num_pages=pages)
+    ctx_b, _ = ctx_for(dtype, list(range(20, n)), page_size=8, num_pages=pages)
+    first = attn.forward(ctx_a, x[:20].to(DEV), cache2)
+    second = attn.forward(ctx_b, x[20:].to(DEV), cache2)
+    check(torch.cat((first, second)), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gated_mlp_part(dtype):
+    mlp = GatedMLP(96, 160, prefix="m")
+    w = fill(mlp, dtype, seed=5)
+    ctx, _ = ctx_for(dtype, [0, 1, 2])
+    x = rnd((3, 96), 6).to(dtype)
+    gu = w["m.gate_up.weight"]
+    want = pm.gated_mlp(x.double(), gu[:160], gu[160:], w["m.down.weight"])
+    check(mlp.forward(ctx, x.to(DEV)), want, dtype)
+    with pytest.raises(ValueError):
+        GatedMLP(8, 8, activation="gelu")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding_and_head(dtype):
+    emb = TokenEmbedding(311, 96, prefix="e")
+    w = fill(emb, dtype, seed=7)["e.weight"]
+    ctx, _ = ctx_for(dtype, [0, 1, 2, 3])
+    ids = torch.tensor([310, 0, 17, 17], dtype=torch.int32, device=DEV)
+    x = emb.forward(ctx, ids)
+    assert x.dtype == dtype and torch.equal(x.double().cpu(), w[[310, 0, 17, 17]])
+    tied = LMHead(311, 96, tied_to=emb, prefix="h")
+    assert tied.param_specs() == {} and tied.weight is emb.params["weight"]
+    logits = tied.forward(ctx, x)
+    assert logits.dtype == torch.float32
+    check(logits, x.double().cpu() @ w.T, dtype)
+    own = LMHead(311, 96, prefix="h")
+    hw = fill(own, dtype, seed=8)["h.weight"]
+    check(own.forward(ctx, x), x.double().cpu() @ hw.T, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_prenorm_block(dtype):
+    norm = PartChoice("rmsnorm", {"size": 64, "eps": 1e-6})
+    block = PreNormBlock(
+        mixer=PartChoice("attention", {"hidden_size": 64, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16,
+                                       "qk_norm": True, "position_encoding": PartChoice("rotary", {"theta": 1e4, "max_positions": 64})}),
+        feed_forward=PartChoice("gated_mlp", {"hidden_size": 64, "intermediate_size": 100}), norm=norm, prefix="model.layers.0")
+    w = fill(block, dtype, seed=9, scale=0.2)
+    n = 21
+    ctx, pages = ctx_for(dtype, list(range(n)))
+    cache = KVBinding(0, torch.zeros((pages, 2, 16, 16), dtype=dtype, device=DEV), torch.zeros((pages, 2, 16, 16), dtype=dtype, device=DEV))
+    x, r = rnd((n, 64), 10).to(dtype), rnd((n, 64), 11)
+    hidden, res = block.forward(ctx, x.to(DEV), r.to(DEV), cache)
+    p = "model.layers.0."
+    summed = x.double() + r.double()
+    h = pm.rms_norm(summed, w[p + "input_layernorm.weight"], 1e-6)
+    qkv = w[p + "self_attn.qkv.weight"]
+    aw = {"q_proj.weight": qkv[:64], "k_proj.weight": qkv[64:96], "v_proj.weight": qkv[96:],
+          "o_proj.weight": w[p + "self_attn.o.weight"], "q_norm.weight": w[p + "self_attn.q_norm.weight"],
+          "k_norm.weight": w[p + "self_attn.k_norm.weight"]}
+    cfg = dict(num_attention_heads=4, num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-6, rope_theta=1e4)
+    a, _ = pm.self_attention(h, torch.arange(n), aw, cfg)
+    h2, res_want = pm.add_rms_norm(a, summed, w[p + "post_attention_layernorm.weight"], 1e-6)
+    gu = w[p + "mlp.gate_up.weight"]
+    want = pm.gated_mlp(h2, gu[:100], gu[100:], w[p + "mlp.down.weight"])
+    check(hidden, want, dtype)
+    check(res, res_want, dtype)
+    # the first block of a model starts the residual stream from its input
+    hidden0, res0 = block.forward(ctx, x.to(DEV), None, cache)
+    h0 = pm.rms_norm(x.double(), w[p + "input_layernorm.weight"], 1e-6)
+    a0, _ = pm.self_attention(h0, torch.arange(n), aw, cfg)
+    _, res0_want = pm.add_rms_norm(a0, x.double(), w[p + "post_attention_layernorm.weight"], 1e-6)
+    check(res0, res0_want, dtype)
+
+
+# ------------------------------------------------------------------ a toy mixer with a state of its own
+
+
+class RunningMeanMixer(Mixer):
+    """y_t = W . mean(x_0 .. x_t): the state of a request is the running sum of its inputs and the
+    number of tokens seen, a fixed size whatever the context."""
+
+    def __init__(self, hidden_size: int, prefix: str = ""):
+        super().__init__(prefix)
+        self.hidden_size = hidden_size
+
+    def param_specs(self):
+        return {"mix.weight": ParamSpec.single("mix.weight", (self.hidden_size, self.hidden_size))}
+
+    def cache_need(self):
+        return StateNeed((self.hidden_size + 1,), torch.float32)
+
+    def forward(self, ctx, x, cache):
+        out = torch.empty_like(x)
+        for start, n, slot in zip(ctx.seq_starts, ctx.seq_lens, ctx.state_slots):
+            state = cache.state[slot]
+            sums = state[:-1] + torch.cumsum(x[start:start + n].float(), dim=0)
+            counts = state[-1] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+            out[start:start + n] = (sums / counts[:, None]).to(x.dtype)
+            state[:-1] = sums[-1]
+            state[-1] = counts[-1]
+        return ctx.ops.linear(out, self.params["mix.weight"])
+
+
+@dataclass(frozen=True)
+class ToyConfig(ModelConfig):
+    num_attention_heads: int = 2
+    head_dim: int = 16
+    intermediate_size: int = 48
+    rms_norm_eps: float = 1e-5
+    model_type: ClassVar[str] = "toy"
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(architecture=raw["architectures"][0], vocab_size=raw["vocab_size"], hidden_size=raw["hidden_size"],
+                   num_hidden_layers=raw["num_hidden_layers"], max_position_embeddings=raw["max_position_embeddings"],
+                   tie_word_embeddings=raw.get("tie_word_embeddings", False), torch_dtype="bfloat16",
+                   bos_token_id=None, eos_token_id=None)
+
+    def to_dict(self):
+        return dict(architectures=[self.architecture], vocab_size=self.vocab_size, hidden_size=self.hidden_size,
+                    num_hidden_layers=self.num_hidden_layers, max_position_embeddings=self.max_position_embeddings,
+                    tie_word_embeddings=self.tie_word_embeddings)
+
+
+def toy_spec(cfg: ToyConfig) -> ModelSpec:
+    norm = PartChoice("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps})
+    ffn = PartChoice("gated_mlp", {"hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size})
+    attn = PartChoice("attention", {"hidden_size": cfg.hidden_size, "num_heads": cfg.num_attention_heads,
+                                    "num_kv_heads": 1, "head_dim": cfg.head_dim,
+                                    "position_encoding": PartChoice("rotary", {"theta": 1e4, "max_positions": cfg.max_position_embeddings})})
+    toy = PartChoice("running_mean", {"hidden_size": cfg.hidden_size})
+    blocks = [PartChoice("prenorm", {"mixer": toy if i % 2 == 0 else attn, "feed_forward": ffn, "norm": norm})
+              for i in range(cfg.num_hidden_layers)]
+    return ModelSpec(cfg.vocab_size, cfg.hidden_size, blocks, norm, max_positions=cfg.max_position_embeddings)
+
+
+def plain_toy_logits(tensors, cfg: ToyConfig, ids):
+    x = tensors["model.embed_tokens.weight"][torch.tensor(ids)]
+    n = len(ids)
+    residual = None
+    for i in range(cfg.num_hidden_layers):
+        p = f"model.layers.{i}."
+        if residual is None:
+            residual, h = x, pm.rms_norm(x, tensors[p + "input_layernorm.weight"], cfg.rms_norm_eps)
+        else:
+            h, residual = pm.add_rms_norm(x, residual, tensors[p + "input_layernorm.weight"], cfg.rms_norm_eps)
+        if i % 2 == 0:
+            mean = torch.cumsum(h, dim=0) / torch.arange(1, n + 1, dtype=h.dtype)[:, None]
+            a = mean @ tensors[p + "self_attn.mix.weight"].T
+        else:
+            t = h.shape[0]
+            q = (h @ tensors[p + "self_attn.q_proj.weight"].T).view(t, cfg.num_attention_heads, cfg.head_dim)
+            k = (h @ tensors[p + "self_attn.k_proj.weight"].T).view(t, 1, cfg.head_dim)
+            v = (h @ tensors[p + "self_attn.v_proj.weight"].T).view(t, 1, cfg.head_dim)
+            cos, sin = pm.rope_angles(torch.arange(t), cfg.head_dim, 1e4)
+            o = pm.causal_attention(pm.rope_neox(q, cos, sin), pm.rope_neox(k, cos, sin), v, cfg.head_dim ** -0.5)
+            a = o.reshape(t, -1) @ tensors[p + "self_attn.o_proj.weight"].T
+        h, residual = pm.add_rms_norm(a, residual, tensors[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps)
+        x = pm.gated_mlp(h, tensors[p + "mlp.gate_proj.weight"], tensors[p + "mlp.up_proj.weight"], tensors[p + "mlp.down_proj.weight"])
+    h, _ = pm.add_rms_norm(x, residual, tensors["model.norm.weight"], cfg.rms_norm_eps)
+    return h @ tensors["lm_head.weight"].T
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype, tmp_path):
+    MIXERS.register("running_mean", RunningMeanMixer)
+    register_architecture("ToyForCausalLM", ToyConfig, toy_spec)
+    try:
+        cfg = ToyConfig.from_dict(dict(architectures=["ToyForCausalLM"], vocab_size=97, hidden_size=40,
+                                       num_hidden_layers=3, max_position_embeddings=96))
+        folder = write_random_model(str(tmp_path / "toy"), cfg, seed=4, std=0.2, norm_std=0.1)
+        from safetensors.torch import load_file
+        tensors = {k: v.double() for k, v in load_file(folder + "/model.safetensors").items()}
+        assert "model.layers.0.self_attn.mix.weight" in tensors and "model.layers.1.self_attn.q_proj.weight" in tensors
+        model, loaded = load_model(folder, dtype=dtype, device=DEV)
+        assert isinstance(loaded, ToyConfig) and isinstance(model.blocks[0].mixer, RunningMeanMixer)
+        core = build_core(model, gpu_ops(), dtype=dtype, device=DEV, page_size=16, num_pages=12, max_num_seqs=3)
+        assert len(core.storage.state_tensors) == 2 and core.storage.state_tensors[0].shape == (3, 41)
+        g = torch.Generator().manual_seed(0)
+        reqs = {r: torch.randint(0, 97, (n,), generator=g).tolist() for r, n in (("a", 50), ("b", 23), ("c", 70))}
+        want = {r: plain_toy_logits(tensors, cfg, ids) for r, ids in reqs.items()}
+        got = {r: {} for r in reqs}
+
+        def step(parts):
+            entries = [StepEntry(r, reqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in parts]
+            logits = core.step(entries)
+            at = 0
+            for r, lo, hi in parts:
+                for pos in range(lo, hi):
+                    got[r][pos] = logits[at].cpu()
+                    at += 1
+
+        step([("a", 0, 20)])
+        step([("a", 20, 21), ("b", 0, 23)])
+        core.close("b")                       # b's slot goes back ...
+        step([("a", 21, 50), ("c", 0, 2)])    # ... and c starts in it with a zeroed state
+        step([("c", 2, 3)])
+        step([("c", 3, 70)])
+        assert core.manager.state_slot("c") == 1
+        tol = 3e-5 if dtype == torch.float32 else 4e-2
+        for r, ids in reqs.items():
+            scale = float(want[r].abs().max())
+            for pos in range(len(ids)):
+                diff = float((got[r][pos].double() - want[r][pos]).abs().max())
+                assert diff <= tol * scale, f"request {r} position {pos}: {diff:.3e} > {tol * scale:.3e}"
+    finally:
+        MIXERS.unregister("running_mean")
+        unregister_architecture("ToyForCausalLM")
