@@ -37,7 +37,8 @@ class StepEntry:
 
 
 class EngineCore:
-    def __init__(self, model, ops, plan: CachePlan, max_num_seqs: int, device, dtype: torch.dtype):
+    def __init__(self, model, ops, plan: CachePlan, max_num_seqs: int, device, dtype: torch.dtype,
+                 graph_sizes: list[int] | None = None, max_model_len: int = 0):
         self.model = model
         self.ops = ops
         self.device = torch.device(device)
@@ -49,6 +50,13 @@ class EngineCore:
         self.max_positions = model.spec.max_positions
         self.steps_run = 0
         self._fresh_slots: list[int] = []      # slots claimed since the last step: zeroed before it runs
+        # decode-only steps replay a captured HIP graph per batch-size bucket (None: always eager)
+        self.graphs = None
+        if graph_sizes:
+            from .graphs import DecodeGraphs
+
+            graphs = DecodeGraphs(self, graph_sizes, max_model_len or self.max_positions)
+            self.graphs = graphs if graphs.usable else None
 
     # ------------------------------------------------------------------ requests
 
@@ -118,8 +126,17 @@ class EngineCore:
         self.storage.reset_state(self._fresh_slots)
         self._fresh_slots = []
 
-        ctx, token_ids, want_rows = self._build(entries, order)
-        logits = self.model.forward(ctx, token_ids, self.storage.bindings, want_rows)
+        cached_now = [self.lengths[e.req_id] for e in entries]
+        if self.graphs is not None and self.graphs.accepts(entries, cached_now):
+            rows = [b for b, e in enumerate(entries) if e.want]
+            logits = None
+            all_logits = self.graphs.run(entries, cached_now)
+            if rows:
+                index = torch.tensor(rows, dtype=torch.long, device=self.device)
+                logits = all_logits.index_select(0, index)
+        else:
+            ctx, token_ids, want_rows = self._build(entries, order)
+            logits = self.model.forward(ctx, token_ids, self.storage.bindings, want_rows)
 
         for e in entries:
             self.lengths[e.req_id] += len(e.tokens)
@@ -225,10 +242,11 @@ def load_model(model_dir: str | None, *, dtype: torch.dtype, device, model_confi
 
 def build_core(model, ops, *, dtype: torch.dtype, device, page_size: int = 16, num_pages: int | None = None,
                budget_bytes: int | None = None, max_num_seqs: int = 4, max_model_len: int = 0,
-               max_num_batched_tokens: int = 0) -> EngineCore:
+               max_num_batched_tokens: int = 0, graph_sizes: list[int] | None = None) -> EngineCore:
     from ..cache.storage import plan_cache
 
     plan = plan_cache(model, page_size, dtype, num_pages=num_pages, budget_bytes=budget_bytes,
                       max_num_seqs=max_num_seqs, max_model_len=max_model_len,
                       max_num_batched_tokens=max_num_batched_tokens)
-    return EngineCore(model, ops, plan, max_num_seqs, device, dtype)
+    return EngineCore(model, ops, plan, max_num_seqs, device, dtype, graph_sizes=graph_sizes,
+                      max_model_len=max_model_len)

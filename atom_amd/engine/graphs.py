@@ -1,0 +1,167 @@
+"""HIP graphs for decode-only steps.
+
+A step in which every request brings one token has the same kernels whatever the
+requests are; only the contents of the step's integer arrays differ.  Such a step is
+captured once per batch-size bucket (the reference captures decode graphs for a list of
+sizes, largest first, atom/model_engine/model_runner.py:3949-4298, sizes from
+atom/model_engine/arg_utils.py:59) and replayed: the arrays live in one static device
+buffer that is overwritten before each replay.  A batch smaller than its bucket is
+padded the reference's way (model_runner.py:2577-2590): padding rows have token 0,
+context length 0 (attention sees no key), cache slot -1 (nothing is written) and
+request index -1.
+
+Buckets are captured on first use.  Every captured graph shares one memory pool.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..kernels.hip import AttentionMeta
+from .context import StepContext
+
+
+class _Captured:
+    def __init__(self, size: int):
+        self.size = size
+        self.graph: torch.cuda.CUDAGraph | None = None
+        self.host: torch.Tensor | None = None      # pinned int32
+        self.dev: torch.Tensor | None = None       # int32, same layout
+        self.logits: torch.Tensor | None = None    # float32 [size, vocab]
+        self.offsets: dict[str, tuple[int, int]] = {}
+        self.copied = torch.cuda.Event()
+        self.copy_pending = False
+
+
+class DecodeGraphs:
+    def __init__(self, core, sizes: list[int], max_model_len: int):
+        self.core = core
+        limit = core.manager.slots.num_slots
+        self.sizes = sorted({int(s) for s in sizes if 0 < int(s) <= limit})
+        self.max_model_len = int(max_model_len)
+        self.widths = [max(1, -(-self.max_model_len // g.page_size)) for g in core.manager.groups]
+        self.captured: dict[int, _Captured] = {}
+        self.pool = None
+        self.replays = 0
+        self.usable = bool(self.sizes) and core.device.type == "cuda" and all(
+            getattr(block.mixer, "graph_safe", False) for block in core.model.blocks)
+
+    def bucket(self, num_seqs: int) -> int | None:
+        for s in self.sizes:
+            if s >= num_seqs:
+                return s
+        return None
+
+    def accepts(self, entries, cached: list[int]) -> bool:
+        if not self.usable or not entries or any(len(e.tokens) != 1 for e in entries):
+            return False
+        if self.bucket(len(entries)) is None:
+            return False
+        return max(cached) + 1 <= self.max_model_len
+
+    # ------------------------------------------------------------------ layout
+
+    def _layout(self, size: int) -> tuple[dict[str, tuple[int, int]], int]:
+        pieces = [("tokens", size), ("positions", size), ("token_seq", size), ("starts", size + 1),
+                  ("context_lens", size), ("want", size)]
+        for gi, width in enumerate(self.widths):
+            pieces += [(f"bt{gi}", size * width), (f"slots{gi}", size)]
+        offsets, cursor = {}, 0
+        for name, n in pieces:
+            offsets[name] = (cursor, n)
+            cursor += (n + 3) // 4 * 4
+        return offsets, cursor
+
+    def _fill(self, cap: _Captured, entries, cached: list[int]) -> None:
+        """Writes the step's arrays into the pinned buffer (padding beyond the entries)."""
+        if cap.copy_pending:
+            cap.copied.synchronize()   # the last copy out of this buffer has finished
+            cap.copy_pending = False
+        host = cap.host.numpy()
+        size, n = cap.size, len(entries)
+        mgr = self.core.manager
+
+        def view(name):
+            off, count = cap.offsets[name]
+            return host[off:off + count]
+
+        tokens, positions, token_seq = view("tokens"), view("positions"), view("token_seq")
+        tokens[:] = 0
+        positions[:] = 0
+        token_seq[:] = -1
+        ctx_lens = view("context_lens")
+        ctx_lens[:] = 0
+        view("starts")[:] = np.arange(size + 1, dtype=np.int32)
+        view("want")[:] = np.arange(size, dtype=np.int32)
+        for b, e in enumerate(entries):
+            tokens[b] = e.tokens[0]
+            positions[b] = cached[b]
+            token_seq[b] = b
+            ctx_lens[b] = cached[b] + 1
+        for gi, width in enumerate(self.widths):
+            bt = view(f"bt{gi}").reshape(size, width)
+            slots = view(f"slots{gi}")
+            slots[:] = -1
+            bt[n:] = 0
+            for b, e in enumerate(entries):
+                table = mgr.block_table(e.req_id, gi)
+                row = np.asarray(table, dtype=np.int32)
+                bt[b, :len(table)] = np.where(row < 0, 0, row)
+                bt[b, len(table):] = 0
+                slots[b] = mgr.slot_mapping(e.req_id, gi, cached[b], 1)[0]
+
+    def _context(self, cap: _Captured):
+        core, size = self.core, cap.size
+
+        def view(name):
+            off, count = cap.offsets[name]
+            return cap.dev[off:off + count]
+
+        ctx = StepContext(ops=core.ops, dtype=core.dtype, device=core.device, num_tokens=size, num_seqs=size,
+                          positions=view("positions"), seq_starts=list(range(size)), seq_lens=[1] * size,
+                          seq_cached=[0] * size, state_slots=[0] * size)
+        for gi, (g, width) in enumerate(zip(core.manager.groups, self.widths)):
+            ctx.attention[gi] = AttentionMeta(
+                token_seq=view("token_seq"), positions=view("positions"),
+                block_tables=view(f"bt{gi}").view(size, width), cu_seqlens_q=view("starts"),
+                context_lens=view("context_lens"), num_seqs=size, num_tokens=size, max_q_len=1,
+                max_context_len=width * g.page_size, page_size=g.page_size, num_prefill=0, prefill_tiles=None)
+            ctx.slot_mappings[gi] = view(f"slots{gi}")
+        return ctx, view("tokens"), view("want")
+
+    # ------------------------------------------------------------------ capture and replay
+
+    def _capture(self, size: int) -> _Captured:
+        core = self.core
+        cap = _Captured(size)
+        cap.offsets, total = self._layout(size)
+        cap.host = torch.zeros(max(total, 4), dtype=torch.int32, pin_memory=True)
+        cap.dev = torch.zeros(max(total, 4), dtype=torch.int32, device=core.device)
+        self._fill(cap, [], [])                       # all padding: the warm-up touches no cache slot
+        cap.dev.copy_(cap.host)
+        ctx, tokens, want = self._context(cap)
+        stream = torch.cuda.Stream(device=core.device)
+        stream.wait_stream(torch.cuda.current_stream(core.device))
+        with torch.cuda.stream(stream):
+            core.model.forward(ctx, tokens, core.storage.bindings, want)   # first-use allocations happen here
+        stream.synchronize()
+        if self.pool is None:
+            self.pool = torch.cuda.graph_pool_handle()
+        cap.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(cap.graph, pool=self.pool, stream=stream):
+            cap.logits = core.model.forward(ctx, tokens, core.storage.bindings, want)
+        self.captured[size] = cap
+        return cap
+
+    def run(self, entries, cached: list[int]) -> torch.Tensor:
+        """Float32 logits [len(entries), vocab] of the entries' single tokens."""
+        size = self.bucket(len(entries))
+        cap = self.captured.get(size) or self._capture(size)
+        self._fill(cap, entries, cached)
+        cap.dev.copy_(cap.host, non_blocking=True)
+        cap.copied.record()
+        cap.copy_pending = True
+        cap.graph.replay()
+        self.replays += 1
+        return cap.logits[:len(entries)]

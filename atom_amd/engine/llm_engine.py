@@ -64,7 +64,8 @@ class LLMEngine:
             num_pages=cfg.num_kvcache_blocks if cfg.num_kvcache_blocks > 0 else None,
             budget_bytes=self._cache_budget() if cfg.num_kvcache_blocks <= 0 else None,
             max_num_seqs=cfg.max_num_seqs, max_model_len=cfg.max_model_len,
-            max_num_batched_tokens=cfg.max_num_batched_tokens)
+            max_num_batched_tokens=cfg.max_num_batched_tokens,
+            graph_sizes=None if cfg.enforce_eager else cfg.cudagraph_capture_sizes)
         self.scheduler = Scheduler(cfg, self.core)
         self.sampler = Sampler(ops, cfg.device)
         self.seqs: dict[int, Sequence] = {}

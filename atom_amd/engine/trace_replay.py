@@ -30,6 +30,7 @@ def main(argv=None) -> int:
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="the most tokens live requests hold at any time (each rounded up to 64)")
     parser.add_argument("--max-requests", type=int, default=8, help="state slots (live requests at a time)")
+    parser.add_argument("--enforce-eager", action="store_true", help="never replay captured HIP graphs")
     args = parser.parse_args(argv)
 
     def say(msg):
@@ -49,7 +50,8 @@ def main(argv=None) -> int:
     model, _ = load_model(args.model, dtype=dtype, device=device, progress=say)
     num_pages = max(1, -(-args.max_tokens // PAGE_SIZE))
     core = build_core(model, ops, dtype=dtype, device=device, page_size=PAGE_SIZE, num_pages=num_pages,
-                      max_num_seqs=args.max_requests)
+                      max_num_seqs=args.max_requests,
+                      graph_sizes=None if args.enforce_eager else [1, 2, 4, 8])
     os.makedirs(args.out, exist_ok=True)
     say(f"ready: {num_pages} pages of {PAGE_SIZE} tokens per group, {args.dtype}")
 

@@ -90,7 +90,11 @@ class HipKernels:
         self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
 
     def workspace(self, name: str, numel: int, dtype=torch.float32) -> torch.Tensor:
-        """A scratch tensor that only grows; one per name."""
+        """A scratch tensor that only grows; one per name.  While a HIP graph is being captured the
+        tensor comes from the graph's own pool instead, so that the graph never holds memory
+        that a later, larger request would free."""
+        if torch.cuda.is_current_stream_capturing():
+            return torch.empty(max(numel, 1), dtype=dtype, device=self.device)
         t = self._ws.get(name)
         if t is None or t.numel() < numel or t.dtype != dtype:
             t = torch.empty(max(numel, 1), dtype=dtype, device=self.device)

@@ -16,6 +16,8 @@ from .base import MIXERS, POSITION_ENCODINGS, KVCacheNeed, Mixer, ParamSpec, Par
 
 
 class GroupedQueryAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool = False, out_bias: bool = False, qk_norm: bool = False, norm_eps: float = 1e-6,
                  scale: float | None = None, window: int | None = None,

@@ -135,6 +135,10 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    #: True when ``forward`` launches the same kernels whatever the batch holds and reads the batch
+    #: only through device arrays of ``ctx``: a decode step of such mixers may be replayed as a HIP graph
+    graph_safe = False
+
     def cache_need(self) -> KVCacheNeed | StateNeed | None:
         return None
 

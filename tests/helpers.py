@@ -47,7 +47,7 @@ def gpu_ops():
 
 
 def make_core(which: str, dtype: str, ops, device: str, num_pages: int = 64, max_num_seqs: int = 8,
-              page_size: int | None = None, stored: str = "bfloat16", order=None):
+              page_size: int | None = None, stored: str = "bfloat16", order=None, graph_sizes=None):
     from atom_amd.engine.core import TORCH_DTYPES, build_core, load_model
 
     tdtype = TORCH_DTYPES[dtype]
@@ -57,4 +57,4 @@ def make_core(which: str, dtype: str, ops, device: str, num_pages: int = 64, max
 
         model.order = [LayerRun(layer, src) for layer, src in order]
     return build_core(model, ops, dtype=tdtype, device=device, page_size=page_size or PAGE[which],
-                      num_pages=num_pages, max_num_seqs=max_num_seqs)
+                      num_pages=num_pages, max_num_seqs=max_num_seqs, graph_sizes=graph_sizes)

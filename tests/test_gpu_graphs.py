@@ -1,0 +1,80 @@
+"""Decode-only steps replayed as HIP graphs: the same traces as the eager engine against the
+plain implementation, and a graph replayed several times, with eager steps of other requests
+between the replays, against the eager result of the same step."""
+
+import pytest
+import torch
+
+import replay
+from helpers import gpu_ops, make_core, oracle_logits, random_ids
+from atom_amd.engine.core import StepEntry
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [40, 17, 90, 128], "B": [1, 9, 71, 200, 130], "C": [50, 600, 95, 257]}
+
+
+def _requests(which):
+    return {f"g{k}": random_ids(which, n, 900 + k) for k, n in enumerate(LENGTHS[which])}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("cut", ["tail", "mixed"])
+def test_graph_cuts_match_plain(which, cut, dtype):
+    requests = _requests(which)
+    oracle = {rid: oracle_logits(which, ids) for rid, ids in requests.items()}
+    steps = replay.tail(requests) if cut == "tail" else replay.mixed(requests, seed=8, decode_tail=20)
+    pages = -(-replay.peak_tokens(steps, 64) // 16)
+    core = make_core(which, dtype, gpu_ops(), "cuda:0", num_pages=pages, page_size=16, graph_sizes=[1, 2, 4])
+    assert core.graphs is not None
+    results = replay.run_in_process(core, steps)
+    assert core.graphs.replays >= 20, "the decode steps of this trace should have been replayed graphs"
+    replay.check(steps, results, requests, oracle, dtype, f"graph/{which}/{cut}/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replays_agree_with_eager(dtype):
+    """Three requests decode together through one graph (bucket 4, one padding row) for 12 steps; in
+    between, another request runs eager prompt portions.  An eager engine runs the same steps."""
+    which = "C"
+    prompts = {f"p{k}": random_ids(which, n, 40 + k) for k, n in enumerate([33, 70, 150])}
+    tails = {rid: random_ids(which, 12, 60 + k) for k, rid in enumerate(prompts)}
+    other = random_ids(which, 200, 99)
+
+    def run(graph_sizes):
+        core = make_core(which, dtype, gpu_ops(), "cuda:0", num_pages=64, page_size=16, graph_sizes=graph_sizes)
+        for rid, ids in prompts.items():
+            core.step([StepEntry(rid, ids, [])])
+        outs = []
+        for t in range(12):
+            logits = core.step([StepEntry(rid, [tails[rid][t]], [0]) for rid in prompts])
+            outs.append(logits.cpu())
+            core.step([StepEntry("other", other[16 * t:16 * t + 16], [15])])   # eager work between replays
+            torch.cuda.synchronize()
+        return outs, core
+
+    eager, _ = run(None)
+    graphed, core = run([4])
+    assert core.graphs.replays == 12
+    scale = max(float(e.abs().max()) for e in eager)
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    for t, (e, g) in enumerate(zip(eager, graphed)):
+        assert torch.isfinite(g).all()
+        assert float((e - g).abs().max()) <= tol * scale, f"replay {t} differs from the eager step"
+
+
+def test_stateful_mixer_is_not_graphed():
+    """A model is replayed only if all its mixers declare themselves graph safe."""
+    from atom_amd.parts.base import Mixer
+
+    assert Mixer.graph_safe is False
+    core = make_core("A", "float32", gpu_ops(), "cuda:0", graph_sizes=[1, 2])
+    assert core.graphs is not None and core.graphs.usable
+    core.model.blocks[0].mixer.graph_safe = False
+    try:
+        from atom_amd.engine.graphs import DecodeGraphs
+
+        assert not DecodeGraphs(core, [1, 2], 128).usable
+    finally:
+        del core.model.blocks[0].mixer.graph_safe
