@@ -103,6 +103,7 @@ class _Request:
     tables: list[list[int]]   # per group: page id per page index, -1 where none is held
     slot: int
     fresh: bool = True        # no step has run for it yet
+    serial: int = 0           # unique per ``open``: a request id that is opened again gets a new one
 
 
 class CacheManager:
@@ -118,6 +119,7 @@ class CacheManager:
         self.pools = [PagePool(g.num_pages) for g in groups]
         self.slots = StateSlots(num_state_slots)
         self._requests: dict[object, _Request] = {}
+        self._opened = 0
 
     # ------------------------------------------------------------------ requests
 
@@ -135,7 +137,8 @@ class CacheManager:
         if req_id in self._requests:
             raise KeyError(f"request {req_id!r} is already open")
         slot = self.slots.claim()
-        self._requests[req_id] = _Request([[] for _ in self.groups], slot)
+        self._opened += 1
+        self._requests[req_id] = _Request([[] for _ in self.groups], slot, serial=self._opened)
         return slot
 
     def close(self, req_id) -> None:
@@ -149,6 +152,10 @@ class CacheManager:
 
     def state_slot(self, req_id) -> int:
         return self._requests[req_id].slot
+
+    def serial(self, req_id) -> int:
+        """A number no other opening of any request has: tells a re-opened request from its earlier life."""
+        return self._requests[req_id].serial
 
     def is_fresh(self, req_id) -> bool:
         return self._requests[req_id].fresh
@@ -179,9 +186,13 @@ class CacheManager:
             if end <= 0:
                 out.append(0)
                 continue
-            first = self._first_page_needed(gi, cached)
             last = (end - 1) // g.page_size
             table = req.tables[gi] if req else []
+            if g.window is None:
+                # nothing is given back before the request ends: the table has no gaps
+                out.append(max(0, last + 1 - len(table)))
+                continue
+            first = self._first_page_needed(gi, cached)
             need = 0
             for idx in range(first, last + 1):
                 if idx >= len(table) or table[idx] < 0:
@@ -203,9 +214,13 @@ class CacheManager:
             end = self._end_for(gi, upto, reserve)
             if end <= 0:
                 continue
-            first = self._first_page_needed(gi, cached)
             last = (end - 1) // g.page_size
             table = req.tables[gi]
+            if g.window is None:
+                while len(table) <= last:
+                    table.append(self.pools[gi].take())
+                continue
+            first = self._first_page_needed(gi, cached)
             while len(table) <= last:
                 table.append(-1)
             for idx in range(first, last + 1):

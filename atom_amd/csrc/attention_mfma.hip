@@ -144,41 +144,56 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
     for (int t = 0; t < DT; ++t) acc[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int k0 = kb; k0 < ke; k0 += 16) {
-    // ---- K block: this lane's key row is k0 + r16 (clamped into the context for addressing)
+  // One block of 16 keys in registers: the K rows as the first product's A operand, the V^T rows
+  // as the second's.  The block after the one being multiplied is loaded ahead of it.
+  struct KVBlock {
+    bf16x8 k32[KX32 ? KCH : 1];
+    s16x4 k16[KX32 ? 1 : KCH];
+    s16x4 v[DT];
+  };
+  auto load_block = [&](int k0, KVBlock& blk) {
+    // this lane's key row is k0 + r16 (clamped into the context for addressing)
     const int krow = min(k0 + r16, ke - 1);
     const int kpage = table[krow / ps];
     const bf16_t* kptr = p.k_cache + (((size_t)kpage * p.hkv + kvh) * ps + (krow % ps)) * D;
-    // ---- V block: this lane's keys are k0 + 4g .. + 3, of output rows d = 16 t + r16
+    // this lane's V keys are k0 + 4g .. + 3, of output rows d = 16 t + r16
     const int vkey = min(k0 + 4 * g, ((ke - 1) & ~3));
     const int vpage = table[vkey / ps];
     const bf16_t* vptr = p.v_cache + (((size_t)vpage * p.hkv + kvh) * D + r16) * (size_t)ps + (vkey % ps);
+    if (KX32) {
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) blk.k32[j] = *reinterpret_cast<const bf16x8*>(kptr + 32 * j + 8 * g);
+    } else {
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) blk.k16[j] = *reinterpret_cast<const s16x4*>(kptr + 16 * j + 4 * g);
+    }
+#pragma unroll
+    for (int t = 0; t < DT; ++t) blk.v[t] = *reinterpret_cast<const s16x4*>(vptr + (size_t)(16 * t) * ps);
+  };
 
+  KVBlock cur, nxt;
+  if (kb < ke) load_block(kb, cur);
+  for (int k0 = kb; k0 < ke; k0 += 16) {
+    if (k0 + 16 < ke) load_block(k0 + 16, nxt);
     f32x4 s[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) s[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (KX32) {
-      bf16x8 kreg[KX32 ? KCH : 1];
-#pragma unroll
-      for (int j = 0; j < KCH; ++j) kreg[j] = *reinterpret_cast<const bf16x8*>(kptr + 32 * j + 8 * g);
 #pragma unroll
       for (int j = 0; j < KCH; ++j)
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-          s[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[j], q32[rt][j], s[rt], 0, 0, 0);
+          s[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k32[j], q32[rt][j], s[rt], 0, 0, 0);
     } else {
-      s16x4 kreg[KX32 ? 1 : KCH];
-#pragma unroll
-      for (int j = 0; j < KCH; ++j) kreg[j] = *reinterpret_cast<const s16x4*>(kptr + 16 * j + 4 * g);
 #pragma unroll
       for (int j = 0; j < KCH; ++j)
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-          s[rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[j], q16[rt][j], s[rt], 0, 0, 0);
+          s[rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(cur.k16[j], q16[rt][j], s[rt], 0, 0, 0);
     }
     s16x4 vreg[DT];
 #pragma unroll
-    for (int t = 0; t < DT; ++t) vreg[t] = *reinterpret_cast<const s16x4*>(vptr + (size_t)(16 * t) * ps);
+    for (int t = 0; t < DT; ++t) vreg[t] = cur.v[t];
 
     // ---- softmax update per row tile; lane holds keys k0 + 4g + i of row r16
 #pragma unroll
@@ -217,6 +232,7 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
         acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg[t], pbits, a, 0, 0, 0);
       }
     }
+    cur = nxt;
   }
 
   // ---- write: lane holds O[row r16][d = 16 t + 4 g + i]
@@ -251,26 +267,55 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
   }
 }
 
-// Merges the partial results of a decode row: one block per (request, head), one thread per d.
-__global__ void attention_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
-                                       bf16_t* __restrict__ out, const int* __restrict__ cu_q, int seq_offset,
-                                       int hq, int d, int parts) {
+// Merges the partial results of a decode row: one block of kMergeGroups waves per (request, head).
+// Lane k of every wave first holds the weight of part k (parts <= 64).  Wave w then adds the
+// parts w, w + kMergeGroups, ... (all their loads are issued together) and the waves' sums are
+// added in wave order through LDS.
+constexpr int kMergeGroups = 8;
+
+__global__ void __launch_bounds__(kMergeGroups* kWave)
+attention_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+                       bf16_t* __restrict__ out, const int* __restrict__ cu_q, int seq_offset,
+                       int hq, int d, int parts) {
+  __shared__ float partial[kMergeGroups][kWave];
   const int seq = blockIdx.y;
   const int head = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
   const size_t base = ((size_t)seq * hq + head) * parts;
-  float top = -INFINITY;
-  for (int k = 0; k < parts; ++k) top = fmaxf(top, ws_ml[(base + k) * 2]);
+  float m = -INFINITY, l = 0.f;
+  if (lane < parts) {
+    m = ws_ml[(base + lane) * 2];
+    l = ws_ml[(base + lane) * 2 + 1];
+  }
+  const float top = wave_max(m);
+  const float w = (m == -INFINITY) ? 0.f : exp2f(m - top);
+  const float den = wave_sum(w * l);
+  const float inv = den > 0.f ? 1.f / den : 0.f;
   const int tok = cu_q[seq + seq_offset];
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    float num = 0.f, den = 0.f;
-    for (int k = 0; k < parts; ++k) {
-      const float m = ws_ml[(base + k) * 2];
-      if (m == -INFINITY) continue;
-      const float w = exp2f(m - top);
-      num += w * ws_o[(base + k) * d + i];
-      den += w * ws_ml[(base + k) * 2 + 1];
+  for (int i0 = 0; i0 < d; i0 += kWave) {
+    const int i = i0 + lane;
+    float o[kWave / kMergeGroups];
+#pragma unroll
+    for (int u = 0; u < kWave / kMergeGroups; ++u) {
+      const int k = wave + u * kMergeGroups;
+      o[u] = (k < parts && i < d) ? ws_o[(base + k) * d + i] : 0.f;
     }
-    out[((size_t)tok * hq + head) * d + i] = static_cast<bf16_t>(den > 0.f ? num / den : 0.f);
+    float num = 0.f;
+#pragma unroll
+    for (int u = 0; u < kWave / kMergeGroups; ++u) {
+      const int k = wave + u * kMergeGroups;
+      num += __shfl(w, k & (kWave - 1), kWave) * o[u];
+    }
+    __syncthreads();   // partial[] of the previous round has been read
+    partial[wave][lane] = num;
+    __syncthreads();
+    if (wave == 0 && i < d) {
+      float total = 0.f;
+#pragma unroll
+      for (int g = 0; g < kMergeGroups; ++g) total += partial[g][lane];
+      out[((size_t)tok * hq + head) * d + i] = static_cast<bf16_t>(total * inv);
+    }
   }
 }
 
@@ -282,7 +327,7 @@ static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
   else if (group <= 32) hipLaunchKernelGGL((attention_mfma_kernel<D, 2, true>), grid, block, 0, stream, p);
   else return ATOM_UNSUPPORTED;
   if (p.parts > 1)
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(p.hq, seqs), dim3(D >= 128 ? 128 : 64), 0, stream, p.ws_o,
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(p.hq, seqs), dim3(kMergeGroups * kWave), 0, stream, p.ws_o,
                        p.ws_ml, p.out, p.cu_q, p.seq_offset, p.hq, D, p.parts);
   return launch_status();
 }
@@ -328,6 +373,7 @@ ATOM_EXPORT int atom_attention_decode(const void* q, const void* k_cache, const 
                                       int window, int parts, float* ws_o, float* ws_ml, hipStream_t stream) {
   if (int st = check_common(hq, hkv, d, page_size, max_blocks)) return st;
   if (seqs < 0 || parts < 1 || seq_offset < 0) return ATOM_BAD_SHAPE;
+  if (parts > kWave) return ATOM_TOO_LARGE;   // the merge keeps one part per lane
   if (parts > 1 && (!ws_o || !ws_ml)) return ATOM_BAD_SHAPE;
   if (seqs > 65535 || hkv > 65535) return ATOM_TOO_LARGE;
   if (seqs == 0) return ATOM_OK;

@@ -75,13 +75,118 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, float* __restrict__ resi
   }
 }
 
+// The same for widths that are a multiple of 8: a thread keeps VPT groups of 8 consecutive
+// elements in registers, all loads of a row are issued at once (16- and 32-byte accesses) and
+// nothing goes through LDS but the reduction.  blockDim.x * 8 * VPT >= width.
+template <typename T>
+struct Vec8;
+template <>
+struct Vec8<float> {
+  float4 a, b;
+  __device__ __forceinline__ void get(float* f) const {
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+  }
+  __device__ __forceinline__ void set(const float* f) {
+    a = make_float4(f[0], f[1], f[2], f[3]);
+    b = make_float4(f[4], f[5], f[6], f[7]);
+  }
+};
+template <>
+struct Vec8<bf16_t> {
+  __attribute__((ext_vector_type(8))) __bf16 v;
+  __device__ __forceinline__ void get(float* f) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = static_cast<float>(v[i]);
+  }
+  __device__ __forceinline__ void set(const float* f) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = static_cast<bf16_t>(f[i]);
+  }
+};
+
+template <typename T, int VPT>
+__global__ void rmsnorm_vec_kernel(const T* __restrict__ x, float* __restrict__ residual,
+                                   const float* __restrict__ weight, T* __restrict__ y,
+                                   const int* __restrict__ rows, int width, float eps, int mode) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  const T* xr = x + (size_t)src * width;
+  float* rr = residual ? residual + (size_t)src * width : nullptr;
+  float vals[VPT][8];
+  float ss = 0.f;
+  Vec8<T> xv[VPT];
+  Vec8<float> rv[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = (threadIdx.x + j * blockDim.x) * 8;
+    if (i < width) {
+      xv[j] = *reinterpret_cast<const Vec8<T>*>(xr + i);
+      if (mode == 2) rv[j] = *reinterpret_cast<const Vec8<float>*>(rr + i);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = (threadIdx.x + j * blockDim.x) * 8;
+    if (i < width) {
+      xv[j].get(vals[j]);
+      if (mode == 2) {
+        float add[8];
+        rv[j].get(add);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vals[j][e] += add[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += vals[j][e] * vals[j][e];
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = rsqrtf(ss / (float)width + eps);
+  T* yr = y + (size_t)r * width;
+  const bool store_residual = mode != 0 && rows == nullptr;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = (threadIdx.x + j * blockDim.x) * 8;
+    if (i < width) {
+      if (store_residual) {
+        Vec8<float> o;
+        o.set(vals[j]);
+        *reinterpret_cast<Vec8<float>*>(rr + i) = o;
+      }
+      Vec8<float> wv = *reinterpret_cast<const Vec8<float>*>(weight + i);
+      float w[8], outv[8];
+      wv.get(w);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) outv[e] = vals[j][e] * inv * w[e];
+      Vec8<T> o;
+      o.set(outv);
+      *reinterpret_cast<Vec8<T>*>(yr + i) = o;
+    }
+  }
+}
+
 ATOM_EXPORT int atom_rmsnorm(const void* x, void* residual, const float* weight, void* y,
                              const int* rows, int dtype, int num_rows, int width, float eps,
                              int mode, hipStream_t stream) {
   if (num_rows < 0 || width <= 0 || mode < 0 || mode > 2) return ATOM_BAD_SHAPE;
   if (mode != 0 && residual == nullptr) return ATOM_BAD_SHAPE;
-  if ((size_t)width * 4 + 64 > 64 * 1024) return ATOM_TOO_LARGE;  // the row is kept in LDS
   if (num_rows == 0) return ATOM_OK;
+  const bool aligned = (((uintptr_t)x | (uintptr_t)y | (uintptr_t)residual | (uintptr_t)weight) & 31) == 0;
+  if (width % 8 == 0 && width <= 8 * 1024 * 4 && aligned) {
+    const int groups = width / 8;
+    int threads = groups <= 64 ? 64 : (groups <= 128 ? 128 : (groups <= 256 ? 256 : (groups <= 512 ? 512 : 1024)));
+    const int vpt = (groups + threads - 1) / threads;
+#define LAUNCH_VEC(V)                                                                                         \
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((rmsnorm_vec_kernel<T, V>), dim3(num_rows), dim3(threads), 0, \
+                                                 stream, (const T*)x, (float*)residual, weight, (T*)y, rows, \
+                                                 width, eps, mode))
+    if (vpt == 1) LAUNCH_VEC(1);
+    else if (vpt == 2) LAUNCH_VEC(2);
+    else LAUNCH_VEC(4);
+#undef LAUNCH_VEC
+    return launch_status();
+  }
+  if ((size_t)width * 4 + 64 > 64 * 1024) return ATOM_TOO_LARGE;  // the row is kept in LDS
   const int threads = width >= 2048 ? 512 : (width >= 512 ? 256 : 64);
   const size_t smem = (size_t)width * 4 + 64;
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((rmsnorm_kernel<T>), dim3(num_rows), dim3(threads), smem,
@@ -103,11 +208,39 @@ __global__ void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ y, int 
   y[idx] = from_f32<T>(g / (1.f + expf(-g)) * u);
 }
 
+// inter % 8 == 0: a thread handles 8 consecutive columns with 16- or 32-byte accesses
+template <typename T>
+__global__ void silu_mul_vec_kernel(const T* __restrict__ x, T* __restrict__ y, int inter, size_t groups) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= groups) return;
+  const int per_row = inter / 8;
+  const size_t row = idx / per_row;
+  const int col = (int)(idx - row * per_row) * 8;
+  const Vec8<T> gv = *reinterpret_cast<const Vec8<T>*>(x + row * 2 * inter + col);
+  const Vec8<T> uv = *reinterpret_cast<const Vec8<T>*>(x + row * 2 * inter + inter + col);
+  float g[8], u[8], o[8];
+  gv.get(g);
+  uv.get(u);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+  Vec8<T> ov;
+  ov.set(o);
+  *reinterpret_cast<Vec8<T>*>(y + row * inter + col) = ov;
+}
+
 ATOM_EXPORT int atom_silu_mul(const void* x, void* y, int dtype, int rows, int inter, hipStream_t stream) {
   if (rows < 0 || inter <= 0) return ATOM_BAD_SHAPE;
   const size_t total = (size_t)rows * inter;
   if (total == 0) return ATOM_OK;
   const int threads = 256;
+  if (inter % 8 == 0 && (((uintptr_t)x | (uintptr_t)y) & 31) == 0) {
+    const size_t groups = total / 8;
+    const size_t blocks = (groups + threads - 1) / threads;
+    if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
+    ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((silu_mul_vec_kernel<T>), dim3((unsigned)blocks), dim3(threads), 0,
+                                                   stream, (const T*)x, (T*)y, inter, groups));
+    return launch_status();
+  }
   const size_t blocks = (total + threads - 1) / threads;
   if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((silu_mul_kernel<T>), dim3((unsigned)blocks), dim3(threads), 0,

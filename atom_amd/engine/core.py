@@ -131,7 +131,9 @@ class EngineCore:
             rows = [b for b, e in enumerate(entries) if e.want]
             logits = None
             all_logits = self.graphs.run(entries, cached_now)
-            if rows:
+            if len(rows) == len(entries):
+                logits = all_logits          # every row wanted: the graph's own output, valid until its next replay
+            elif rows:
                 index = torch.tensor(rows, dtype=torch.long, device=self.device)
                 logits = all_logits.index_select(0, index)
         else:

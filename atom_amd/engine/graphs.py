@@ -32,6 +32,9 @@ class _Captured:
         self.offsets: dict[str, tuple[int, int]] = {}
         self.copied = torch.cuda.Event()
         self.copy_pending = False
+        # what the pinned buffer holds per row and group: (the request's serial, pages written), so that a
+        # request that keeps its row only has its new pages written
+        self.row_state: list[list[tuple | None]] = []
 
 
 class DecodeGraphs:
@@ -99,17 +102,32 @@ class DecodeGraphs:
             positions[b] = cached[b]
             token_seq[b] = b
             ctx_lens[b] = cached[b] + 1
+        if not cap.row_state:
+            cap.row_state = [[None] * size for _ in self.widths]
         for gi, width in enumerate(self.widths):
             bt = view(f"bt{gi}").reshape(size, width)
             slots = view(f"slots{gi}")
             slots[:] = -1
-            bt[n:] = 0
+            page_size = mgr.groups[gi].page_size
+            windowed = mgr.groups[gi].window is not None
+            state = cap.row_state[gi]
             for b, e in enumerate(entries):
                 table = mgr.block_table(e.req_id, gi)
-                row = np.asarray(table, dtype=np.int32)
-                bt[b, :len(table)] = np.where(row < 0, 0, row)
-                bt[b, len(table):] = 0
-                slots[b] = mgr.slot_mapping(e.req_id, gi, cached[b], 1)[0]
+                page = table[cached[b] // page_size]
+                if page < 0:
+                    raise AssertionError(f"request {e.req_id!r}: position {cached[b]} has no page")
+                slots[b] = page * page_size + cached[b] % page_size
+                held = state[b]
+                serial = mgr.serial(e.req_id)
+                if not windowed and held is not None and held[0] == serial and held[1] <= len(table):
+                    if held[1] < len(table):     # pages appended since the row was last written
+                        bt[b, held[1]:len(table)] = table[held[1]:]
+                else:
+                    row = np.asarray(table, dtype=np.int32)
+                    bt[b, :len(table)] = np.where(row < 0, 0, row)
+                    bt[b, len(table):] = 0
+                state[b] = (serial, len(table))
+            # rows beyond the entries keep what they had: their context length is 0, nothing reads them
 
     def _context(self, cap: _Captured):
         core, size = self.core, cap.size

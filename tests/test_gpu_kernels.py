@@ -43,7 +43,7 @@ def test_embedding(tdtype, odtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width", [16, 136, 4096, 5000])
+@pytest.mark.parametrize("width", [16, 136, 4096, 5000, 5001, 20000])
 @pytest.mark.parametrize("mode", ["plain", "init", "add"])
 def test_rmsnorm(dtype, width, mode):
     rows = 7
@@ -77,15 +77,16 @@ def test_rmsnorm_rows(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_silu_mul(dtype):
-    x = rnd((5, 2 * 333), dtype, 7, 2.0)
-    out = torch.empty((5, 333), dtype=dtype, device=DEV)
+@pytest.mark.parametrize("inter", [333, 200, 1032])
+def test_silu_mul(dtype, inter):
+    x = rnd((5, 2 * inter), dtype, 7, 2.0)
+    out = torch.empty((5, inter), dtype=dtype, device=DEV)
     gpu_ops().silu_mul(x.to(DEV), out)
-    want = torch.empty((5, 333), dtype=dtype)
+    want = torch.empty((5, inter), dtype=dtype)
     PLAIN.silu_mul(x, want)
     close(out, want, dtype)
-    swapped = torch.cat((x[:, 333:], x[:, :333]), dim=1)
-    other = torch.empty((5, 333), dtype=dtype)
+    swapped = torch.cat((x[:, inter:], x[:, :inter]), dim=1)
+    other = torch.empty((5, inter), dtype=dtype)
     PLAIN.silu_mul(swapped, other)
     assert (other.float() - want.float()).abs().max() > 0.1, "gate and up must not be interchangeable"
 
@@ -348,8 +349,9 @@ def test_kernels_refuse_what_they_cannot_take():
     with pytest.raises(KernelError):
         ops.rmsnorm(x.cpu(), torch.ones(64), 1e-6, torch.empty_like(x.cpu()))
     with pytest.raises(KernelError):
-        ops.rmsnorm(torch.zeros((2, 20000), device=DEV), torch.ones(20000, device=DEV), 1e-6,
-                    torch.zeros((2, 20000), device=DEV))
+        # an odd width goes through LDS, which holds 16 K floats
+        ops.rmsnorm(torch.zeros((2, 20001), device=DEV), torch.ones(20001, device=DEV), 1e-6,
+                    torch.zeros((2, 20001), device=DEV))
     with pytest.raises(KernelError):
         ops.silu_mul(torch.zeros((2, 7), device=DEV), torch.zeros((2, 3), device=DEV))
     with pytest.raises(KernelError):
