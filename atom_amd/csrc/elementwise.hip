@@ -6,6 +6,21 @@
 // the residual stream and norm weights are always float32.
 #include "common.h"
 
+// An input that is still a sum: `splits` float32 slices [rows, width] `stride` elements apart, as the
+// skinny matrix product leaves them when it cuts K, plus an optional bias over the width.  Readers
+// add the slices in slice order.  `partial == nullptr`: the input is an ordinary tensor.
+struct SplitSum {
+  const float* partial;
+  const float* bias;
+  size_t stride;
+  int splits;
+  __device__ __forceinline__ float at(size_t offset, int col) const {
+    float v = 0.f;
+    for (int s = 0; s < splits; ++s) v += partial[(size_t)s * stride + offset];
+    return bias ? v + bias[col] : v;
+  }
+};
+
 // ------------------------------------------------------------------ embedding
 
 template <typename TT, typename TO>
@@ -49,7 +64,7 @@ ATOM_EXPORT int atom_embedding(const void* table, int table_dtype, const int* id
 template <typename T>
 __global__ void rmsnorm_kernel(const T* __restrict__ x, float* __restrict__ residual,
                                const float* __restrict__ weight, T* __restrict__ y,
-                               const int* __restrict__ rows, int width, float eps, int mode) {
+                               const int* __restrict__ rows, int width, float eps, int mode, SplitSum xsum) {
   extern __shared__ float smem[];  // width floats + 16 for the reduction
   float* vals = smem;
   float* scratch = smem + width;
@@ -59,7 +74,7 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, float* __restrict__ resi
   float* rr = residual ? residual + (size_t)src * width : nullptr;
   float ss = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    float v = to_f32(xr[i]);
+    float v = xsum.partial ? xsum.at((size_t)src * width + i, i) : to_f32(xr[i]);
     if (mode == 2) v += rr[i];
     vals[i] = v;
     ss += v * v;
@@ -107,7 +122,7 @@ struct Vec8<bf16_t> {
 template <typename T, int VPT>
 __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, float* __restrict__ residual,
                                    const float* __restrict__ weight, T* __restrict__ y,
-                                   const int* __restrict__ rows, int width, float eps, int mode) {
+                                   const int* __restrict__ rows, int width, float eps, int mode, SplitSum xsum) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
@@ -121,7 +136,7 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, float* __restrict__ 
   for (int j = 0; j < VPT; ++j) {
     const int i = (threadIdx.x + j * blockDim.x) * 8;
     if (i < width) {
-      xv[j] = *reinterpret_cast<const Vec8<T>*>(xr + i);
+      if (!xsum.partial) xv[j] = *reinterpret_cast<const Vec8<T>*>(xr + i);
       if (mode == 2) rv[j] = *reinterpret_cast<const Vec8<float>*>(rr + i);
     }
   }
@@ -129,7 +144,25 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, float* __restrict__ 
   for (int j = 0; j < VPT; ++j) {
     const int i = (threadIdx.x + j * blockDim.x) * 8;
     if (i < width) {
-      xv[j].get(vals[j]);
+      if (xsum.partial) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vals[j][e] = 0.f;
+        const float* base = xsum.partial + (size_t)src * width + i;
+        for (int sp = 0; sp < xsum.splits; ++sp) {
+          float part[8];
+          reinterpret_cast<const Vec8<float>*>(base + (size_t)sp * xsum.stride)->get(part);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) vals[j][e] += part[e];
+        }
+        if (xsum.bias) {
+          float part[8];
+          reinterpret_cast<const Vec8<float>*>(xsum.bias + i)->get(part);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) vals[j][e] += part[e];
+        }
+      } else {
+        xv[j].get(vals[j]);
+      }
       if (mode == 2) {
         float add[8];
         rv[j].get(add);
@@ -165,13 +198,19 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, float* __restrict__ 
   }
 }
 
+// `x_partial` (with `x_splits` slices `x_stride` elements apart and an optional `x_bias`) stands for x
+// when x is still a sum of slices; x itself is then not read.
 ATOM_EXPORT int atom_rmsnorm(const void* x, void* residual, const float* weight, void* y,
                              const int* rows, int dtype, int num_rows, int width, float eps,
-                             int mode, hipStream_t stream) {
+                             int mode, const float* x_partial, int x_splits, long x_stride,
+                             const float* x_bias, hipStream_t stream) {
   if (num_rows < 0 || width <= 0 || mode < 0 || mode > 2) return ATOM_BAD_SHAPE;
   if (mode != 0 && residual == nullptr) return ATOM_BAD_SHAPE;
+  if (x_partial ? (x_splits < 1 || x_stride < 0) : x == nullptr) return ATOM_BAD_SHAPE;
   if (num_rows == 0) return ATOM_OK;
-  const bool aligned = (((uintptr_t)x | (uintptr_t)y | (uintptr_t)residual | (uintptr_t)weight) & 31) == 0;
+  const SplitSum xsum{x_partial, x_partial ? x_bias : nullptr, (size_t)x_stride, x_splits};
+  const bool aligned = (((uintptr_t)x | (uintptr_t)y | (uintptr_t)residual | (uintptr_t)weight |
+                         (uintptr_t)x_partial | (uintptr_t)x_bias) & 31) == 0 && (!x_partial || x_stride % 8 == 0);
   if (width % 8 == 0 && width <= 8 * 1024 * 4 && aligned) {
     const int groups = width / 8;
     int threads = groups <= 64 ? 64 : (groups <= 128 ? 128 : (groups <= 256 ? 256 : (groups <= 512 ? 512 : 1024)));
@@ -179,7 +218,7 @@ ATOM_EXPORT int atom_rmsnorm(const void* x, void* residual, const float* weight,
 #define LAUNCH_VEC(V)                                                                                         \
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((rmsnorm_vec_kernel<T, V>), dim3(num_rows), dim3(threads), 0, \
                                                  stream, (const T*)x, (float*)residual, weight, (T*)y, rows, \
-                                                 width, eps, mode))
+                                                 width, eps, mode, xsum))
     if (vpt == 1) LAUNCH_VEC(1);
     else if (vpt == 2) LAUNCH_VEC(2);
     else LAUNCH_VEC(4);
@@ -191,36 +230,61 @@ ATOM_EXPORT int atom_rmsnorm(const void* x, void* residual, const float* weight,
   const size_t smem = (size_t)width * 4 + 64;
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((rmsnorm_kernel<T>), dim3(num_rows), dim3(threads), smem,
                                                  stream, (const T*)x, (float*)residual, weight, (T*)y,
-                                                 rows, width, eps, mode));
+                                                 rows, width, eps, mode, xsum));
   return launch_status();
 }
 
 // ------------------------------------------------------------------ SiLU(gate) * up
 
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ y, int inter, size_t total) {
+__global__ void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ y, int inter, size_t total, SplitSum xsum) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t row = idx / inter;
   const int col = (int)(idx - row * inter);
-  const float g = to_f32(x[row * 2 * inter + col]);
-  const float u = to_f32(x[row * 2 * inter + inter + col]);
+  const float g = xsum.partial ? xsum.at(row * 2 * inter + col, col) : to_f32(x[row * 2 * inter + col]);
+  const float u = xsum.partial ? xsum.at(row * 2 * inter + inter + col, inter + col)
+                               : to_f32(x[row * 2 * inter + inter + col]);
   y[idx] = from_f32<T>(g / (1.f + expf(-g)) * u);
 }
 
 // inter % 8 == 0: a thread handles 8 consecutive columns with 16- or 32-byte accesses
 template <typename T>
-__global__ void silu_mul_vec_kernel(const T* __restrict__ x, T* __restrict__ y, int inter, size_t groups) {
+__global__ void silu_mul_vec_kernel(const T* __restrict__ x, T* __restrict__ y, int inter, size_t groups,
+                                    SplitSum xsum) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= groups) return;
   const int per_row = inter / 8;
   const size_t row = idx / per_row;
   const int col = (int)(idx - row * per_row) * 8;
-  const Vec8<T> gv = *reinterpret_cast<const Vec8<T>*>(x + row * 2 * inter + col);
-  const Vec8<T> uv = *reinterpret_cast<const Vec8<T>*>(x + row * 2 * inter + inter + col);
   float g[8], u[8], o[8];
-  gv.get(g);
-  uv.get(u);
+  if (xsum.partial) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) g[e] = u[e] = 0.f;
+    const float* base = xsum.partial + row * 2 * inter + col;
+    for (int sp = 0; sp < xsum.splits; ++sp) {
+      float a[8], b[8];
+      reinterpret_cast<const Vec8<float>*>(base + (size_t)sp * xsum.stride)->get(a);
+      reinterpret_cast<const Vec8<float>*>(base + (size_t)sp * xsum.stride + inter)->get(b);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        g[e] += a[e];
+        u[e] += b[e];
+      }
+    }
+    if (xsum.bias) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        g[e] += xsum.bias[col + e];
+        u[e] += xsum.bias[inter + col + e];
+      }
+    }
+  } else {
+    const Vec8<T> gv = *reinterpret_cast<const Vec8<T>*>(x + row * 2 * inter + col);
+    const Vec8<T> uv = *reinterpret_cast<const Vec8<T>*>(x + row * 2 * inter + inter + col);
+    gv.get(g);
+    uv.get(u);
+  }
 #pragma unroll
   for (int e = 0; e < 8; ++e) o[e] = g[e] / (1.f + expf(-g[e])) * u[e];
   Vec8<T> ov;
@@ -228,23 +292,29 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ x, T* __restrict__ y, 
   *reinterpret_cast<Vec8<T>*>(y + row * inter + col) = ov;
 }
 
-ATOM_EXPORT int atom_silu_mul(const void* x, void* y, int dtype, int rows, int inter, hipStream_t stream) {
+// `x_partial` (slices `x_stride` apart, optional `x_bias`) stands for x when x is still a sum of slices;
+// `dtype` is then the type of y.
+ATOM_EXPORT int atom_silu_mul(const void* x, void* y, int dtype, int rows, int inter, const float* x_partial,
+                              int x_splits, long x_stride, const float* x_bias, hipStream_t stream) {
   if (rows < 0 || inter <= 0) return ATOM_BAD_SHAPE;
+  if (x_partial ? (x_splits < 1 || x_stride < 0) : x == nullptr) return ATOM_BAD_SHAPE;
   const size_t total = (size_t)rows * inter;
   if (total == 0) return ATOM_OK;
+  const SplitSum xsum{x_partial, x_partial ? x_bias : nullptr, (size_t)x_stride, x_splits};
   const int threads = 256;
-  if (inter % 8 == 0 && (((uintptr_t)x | (uintptr_t)y) & 31) == 0) {
+  if (inter % 8 == 0 && (((uintptr_t)x | (uintptr_t)y | (uintptr_t)x_partial) & 31) == 0 &&
+      (!x_partial || x_stride % 8 == 0)) {
     const size_t groups = total / 8;
     const size_t blocks = (groups + threads - 1) / threads;
     if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
     ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((silu_mul_vec_kernel<T>), dim3((unsigned)blocks), dim3(threads), 0,
-                                                   stream, (const T*)x, (T*)y, inter, groups));
+                                                   stream, (const T*)x, (T*)y, inter, groups, xsum));
     return launch_status();
   }
   const size_t blocks = (total + threads - 1) / threads;
   if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((silu_mul_kernel<T>), dim3((unsigned)blocks), dim3(threads), 0,
-                                                 stream, (const T*)x, (T*)y, inter, total));
+                                                 stream, (const T*)x, (T*)y, inter, total, xsum));
   return launch_status();
 }
 
@@ -267,12 +337,15 @@ __global__ void qk_norm_rope_kv_write_kernel(
     const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ slots,
-    int hq, int hkv, int d, int rotary_dim, int page_size, float eps, int write_kv) {
+    int hq, int hkv, int d, int rotary_dim, int page_size, float eps, int write_kv, SplitSum xsum) {
   const int t = blockIdx.x;
   const int head = blockIdx.y;  // 0..hq-1 q, then hkv k heads, then hkv v heads
   const int lane = threadIdx.x;
   const int row_width = (hq + 2 * hkv) * d;
   const T* src = qkv + (size_t)t * row_width + (size_t)head * d;
+  const size_t src_off = (size_t)t * row_width + (size_t)head * d;
+  // element i of this head's input: the tensor, or the sum of its slices
+  auto in = [&](int i) -> float { return xsum.partial ? xsum.at(src_off + i, head * d + i) : to_f32(src[i]); };
   const bool is_q = head < hq;
   const bool is_k = !is_q && head < hq + hkv;
   const int kv_head = is_q ? 0 : (is_k ? head - hq : head - hq - hkv);
@@ -288,7 +361,7 @@ __global__ void qk_norm_rope_kv_write_kernel(
 
   if (!is_q && !is_k) {  // value head: plain scatter into the transposed page
     T* dst = v_cache + ((size_t)page * hkv + kv_head) * (size_t)d * page_size + off;
-    for (int i = lane; i < d; i += kWave) dst[(size_t)i * page_size] = src[i];
+    for (int i = lane; i < d; i += kWave) dst[(size_t)i * page_size] = from_f32<T>(in(i));
     return;
   }
 
@@ -297,7 +370,7 @@ __global__ void qk_norm_rope_kv_write_kernel(
   if (weight) {
     float ss = 0.f;
     for (int i = lane; i < d; i += kWave) {
-      const float v = to_f32(src[i]);
+      const float v = in(i);
       ss += v * v;
     }
     ss = wave_sum(ss);
@@ -310,8 +383,8 @@ __global__ void qk_norm_rope_kv_write_kernel(
   const float* cs = cos_table + (size_t)pos * half;
   const float* sn = sin_table + (size_t)pos * half;
   for (int j = lane; j < half; j += kWave) {
-    float x1 = to_f32(src[j]);
-    float x2 = to_f32(src[j + half]);
+    float x1 = in(j);
+    float x2 = in(j + half);
     if (weight) {
       x1 = x1 * inv * weight[j];
       x2 = x2 * inv * weight[j + half];
@@ -321,7 +394,7 @@ __global__ void qk_norm_rope_kv_write_kernel(
     dst[j + half] = from_f32<T>(x2 * c + x1 * s);
   }
   for (int i = rotary_dim + lane; i < d; i += kWave) {  // the part that is not rotated
-    float v = to_f32(src[i]);
+    float v = in(i);
     if (weight) v = v * inv * weight[i];
     dst[i] = from_f32<T>(v);
   }
@@ -331,8 +404,10 @@ ATOM_EXPORT int atom_qk_norm_rope_kv_write(
     const void* qkv, void* q_out, void* k_cache, void* v_cache, const float* q_weight, const float* k_weight,
     const float* cos_table, const float* sin_table, const int* positions, const int* slots, int dtype,
     int tokens, int hq, int hkv, int d, int rotary_dim, int page_size, float eps, int write_kv,
-    hipStream_t stream) {
+    const float* x_partial, int x_splits, long x_stride, const float* x_bias, hipStream_t stream) {
   if (tokens < 0 || hq <= 0 || hkv <= 0 || d <= 0 || page_size <= 0) return ATOM_BAD_SHAPE;
+  if (x_partial ? (x_splits < 1 || x_stride < 0) : qkv == nullptr) return ATOM_BAD_SHAPE;
+  const SplitSum xsum{x_partial, x_partial ? x_bias : nullptr, (size_t)x_stride, x_splits};
   if (rotary_dim < 0 || rotary_dim > d || (rotary_dim & 1)) return ATOM_BAD_SHAPE;
   if (rotary_dim > 0 && (!cos_table || !sin_table || !positions)) return ATOM_BAD_SHAPE;
   if (write_kv && (!k_cache || !v_cache || !slots)) return ATOM_BAD_SHAPE;
@@ -342,6 +417,6 @@ ATOM_EXPORT int atom_qk_norm_rope_kv_write(
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<T>), grid, block, 0, stream,
                                                  (const T*)qkv, (T*)q_out, (T*)k_cache, (T*)v_cache, q_weight,
                                                  k_weight, cos_table, sin_table, positions, slots, hq, hkv, d,
-                                                 rotary_dim, page_size, eps, write_kv));
+                                                 rotary_dim, page_size, eps, write_kv, xsum));
   return launch_status();
 }

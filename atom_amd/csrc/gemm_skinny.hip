@@ -1,0 +1,265 @@
+// y[M, N] = x[M, K] * w[N, K]^T (+ bias) for few rows (M <= 64), bfloat16 operands,
+// float32 accumulation on the matrix cores.  This is the decode-step product: the
+// weight matrix is streamed from memory once and the work is bound by that stream.
+//
+// A block of four waves owns 64 rows of w (64 output columns) and a slice of K; each
+// wave owns 16 of the rows.  The weights are the A operand of v_mfma_f32_16x16x32_bf16
+// and are loaded from memory straight into the operand layout (lane (r, g) holds
+// w[row r][k + 8 g .. k + 8 g + 7], 16 bytes), a chunk of 256 k ahead of the chunk being
+// multiplied.  x is the B operand; the block's slice of it is staged in LDS and shared
+// by the four waves, so x is read from the cache hierarchy once per 64 rows of w.
+// Blocks that are neighbours in the grid read neighbouring slices of the same rows.
+//
+// When N / 64 blocks would not fill the chip, K is cut into `splits` slices and every
+// block writes its partial tile to partial[split][m][n] (float32).  Whoever reads the
+// product next adds the slices in slice order: the norm, the rotation kernel, SiLU-mul,
+// or atom_splitk_reduce.  The sum has one fixed order, so a row's result does not
+// depend on its batch.
+//
+// Epilogues when K is not cut: plain (bias optional, bfloat16 or float32 out), or
+// SiLU-gate: w holds `inter` gate rows then `inter` up rows, a block owns 32 columns of
+// each, and writes silu(gate) * up [M, inter].
+//
+// Needs K % 8 == 0 (16-byte loads).  Any N, any M <= 64.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+
+struct SkinnyParams {
+  const bf16_t* x;     // [m, k]
+  const bf16_t* w;     // [n, k]  (gate: [2 * inter, k])
+  const float* bias;   // [n] or null (only used when splits == 1)
+  void* y;             // splits == 1: [m, n] bfloat16 or float32 (gate: [m, inter] bfloat16)
+  float* partial;      // splits > 1: [splits, m, n]
+  int m, n, k, inter, out_f32, splits, tiles, kslice, xk;
+};
+
+constexpr int kSkinnyRows = 64;    // rows of w per block
+constexpr int kSkinnyChunk = 256;  // k elements per chunk
+constexpr int kSkinnyU = kSkinnyChunk / 32;
+constexpr int kSkinnyLds = 64 * 1024;
+
+template <int MT, bool GATE>
+__global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
+  constexpr int U = kSkinnyU;
+  extern __shared__ __attribute__((aligned(16))) char smem[];   // x slice; later the float32 tile
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int r16 = lane & 15;
+  const int g = lane >> 4;
+  const int k = p.k;
+  const int tile = blockIdx.x / p.splits;
+  const int split = blockIdx.x - tile * p.splits;
+  const int k_begin = split * p.kslice;
+  const int k_end = min(k, k_begin + p.kslice);
+  const int xrow_bytes = p.xk * 2 + 16;   // 16 bytes of padding: rows start 4 banks apart
+
+  // the row of w this lane streams, and the output column it stands for
+  int wrow;
+  if (GATE) {
+    const int col = tile * 32 + (wave & 1) * 16 + r16;
+    wrow = min(col, p.inter - 1) + (wave >= 2 ? p.inter : 0);
+  } else {
+    wrow = min(tile * kSkinnyRows + wave * 16 + r16, p.n - 1);
+  }
+  const bf16_t* wp = p.w + (size_t)wrow * k + 8 * g;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  int xrow[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) xrow[t] = min(16 * t + r16, p.m - 1) * xrow_bytes + 16 * g;
+
+  bf16x8 a_next[U];
+  auto load_a = [&](int kc) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = kc + 32 * u;
+      a_next[u] = (kk + 8 * g < k) ? *reinterpret_cast<const bf16x8*>(wp + kk) : zero;
+    }
+  };
+  if (k_begin < k_end) load_a(k_begin);
+
+  for (int x0 = k_begin; x0 < k_end; x0 += p.xk) {
+    const int x1 = min(k_end, x0 + p.xk);
+    const int pieces = (x1 - x0 + 7) / 8;    // 16-byte pieces per row
+    if (x0 != k_begin) __syncthreads();      // the previous slice of x has been read
+    for (int q = tid; q < p.m * pieces; q += 256) {
+      const int row = q / pieces, piece = q - row * pieces;
+      const int kk = x0 + 8 * piece;
+      const bf16x8 v = kk < k ? *reinterpret_cast<const bf16x8*>(p.x + (size_t)row * k + kk) : zero;
+      *reinterpret_cast<bf16x8*>(smem + row * xrow_bytes + piece * 16) = v;
+    }
+    // a chunk that reaches beyond K reads pieces the loop above did not write: zero them
+    const int padded = ((x1 - x0 + kSkinnyChunk - 1) / kSkinnyChunk) * (kSkinnyChunk / 8);
+    for (int q = tid; q < p.m * (padded - pieces); q += 256) {
+      const int row = q / (padded - pieces), piece = pieces + q - row * (padded - pieces);
+      *reinterpret_cast<bf16x8*>(smem + row * xrow_bytes + piece * 16) = zero;
+    }
+    __syncthreads();
+    for (int kc = x0; kc < x1; kc += kSkinnyChunk) {
+      bf16x8 a[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) a[u] = a_next[u];
+      if (kc + kSkinnyChunk < k_end) load_a(kc + kSkinnyChunk);
+      const char* xb = smem + (kc - x0) * 2;
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const bf16x8 bv = *reinterpret_cast<const bf16x8*>(xb + xrow[t] + 64 * u);
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc[t], 0, 0, 0);
+        }
+    }
+  }
+
+  // ---- the block's float32 tile [m][64] through LDS: lane holds rows m = 16 t + r16, columns 16 wave + 4 g + i
+  __syncthreads();
+  float* tile_f = reinterpret_cast<float*>(smem);   // [m][65]
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = 16 * t + r16;
+    if (m < p.m) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) tile_f[m * (kSkinnyRows + 1) + 16 * wave + 4 * g + i] = acc[t][i];
+    }
+  }
+  __syncthreads();
+
+  if (p.splits > 1) {
+    float* mine = p.partial + (size_t)split * p.m * p.n;
+    for (int item = tid; item < p.m * kSkinnyRows; item += 256) {
+      const int m = item >> 6, c = item & 63;
+      int col;
+      if (GATE) {
+        col = tile * 32 + (c & 31);
+        if (col >= p.inter) continue;
+        col += (c >= 32 ? p.inter : 0);
+      } else {
+        col = tile * kSkinnyRows + c;
+        if (col >= p.n) continue;
+      }
+      mine[(size_t)m * p.n + col] = tile_f[m * (kSkinnyRows + 1) + c];
+    }
+    return;
+  }
+  if (GATE) {
+    for (int item = tid; item < p.m * 32; item += 256) {
+      const int m = item >> 5, c = item & 31;
+      const int col = tile * 32 + c;
+      if (col >= p.inter) continue;
+      float gv = tile_f[m * (kSkinnyRows + 1) + c];
+      float uv = tile_f[m * (kSkinnyRows + 1) + 32 + c];
+      if (p.bias) {
+        gv += p.bias[col];
+        uv += p.bias[p.inter + col];
+      }
+      reinterpret_cast<bf16_t*>(p.y)[(size_t)m * p.inter + col] = from_f32<bf16_t>(gv / (1.f + expf(-gv)) * uv);
+    }
+  } else {
+    for (int item = tid; item < p.m * kSkinnyRows; item += 256) {
+      const int m = item >> 6, c = item & 63;
+      const int col = tile * kSkinnyRows + c;
+      if (col >= p.n) continue;
+      const float v = tile_f[m * (kSkinnyRows + 1) + c] + (p.bias ? p.bias[col] : 0.f);
+      if (p.out_f32) reinterpret_cast<float*>(p.y)[(size_t)m * p.n + col] = v;
+      else reinterpret_cast<bf16_t*>(p.y)[(size_t)m * p.n + col] = from_f32<bf16_t>(v);
+    }
+  }
+}
+
+// y[m, n] = sum over splits of partial[s][m][n] (+ bias), in slice order.
+template <typename TY>
+__global__ void splitk_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ bias,
+                                     TY* __restrict__ y, size_t total, int n, int splits) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  float s = 0.f;
+  for (int sp = 0; sp < splits; ++sp) s += partial[(size_t)sp * total + idx];
+  if (bias) s += bias[idx % n];
+  y[idx] = from_f32<TY>(s);
+}
+
+static int skinny_tiles(int n, int gate) { return gate ? (n + 31) / 32 : (n + kSkinnyRows - 1) / kSkinnyRows; }
+
+// How K is cut: enough blocks to keep about a thousand in flight, slices a multiple of 512.
+static void skinny_plan(int m, int tiles, int k, int* splits, int* kslice, int* xk) {
+  const int units = (k + 511) / 512;
+  int s = (1024 + tiles - 1) / tiles;
+  s = max(1, min(s, min(units, 32)));
+  const int per = (units + s - 1) / s;           // units of 512 per slice
+  *kslice = per * 512;
+  *splits = (units + per - 1) / per;
+  int cap = (kSkinnyLds - 64) / m / 2 - 8;       // k elements of one row of x that fit
+  cap = max(kSkinnyChunk, cap / kSkinnyChunk * kSkinnyChunk);
+  *xk = min(*kslice, cap);
+}
+
+// 1 if the skinny kernel takes this product.
+ATOM_EXPORT int atom_gemm_skinny_supports(int m, int n, int k) {
+  return m >= 1 && m <= 64 && n >= 1 && k >= 8 && k % 8 == 0;
+}
+
+// Into how many slices atom_gemm_skinny cuts K for this product (1: it writes y itself).
+ATOM_EXPORT int atom_gemm_skinny_splits(int m, int n, int k, int gate) {
+  int splits, kslice, xk;
+  skinny_plan(max(m, 1), skinny_tiles(n, gate), k, &splits, &kslice, &xk);
+  return splits;
+}
+
+// gate == 0: x w^T, n columns.  gate == 1: w is [2 n, k] (n gate rows, then n up rows).
+// With atom_gemm_skinny_splits(...) == 1 the result goes to y: [m, n] bfloat16 (or float32 with
+// out_f32; gate: silu(x wg^T) * (x wu^T), bfloat16), bias added.  Otherwise y is not touched, bias
+// is not used and partial[splits][m][columns] receives the slices' products (columns = 2 n for gate).
+ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias, void* y, float* partial,
+                                 int m, int n, int k, int out_f32, int gate, hipStream_t stream) {
+  if (m < 0 || n <= 0 || k <= 0) return ATOM_BAD_SHAPE;
+  if (m > 64 || k % 8) return ATOM_UNSUPPORTED;
+  if (gate && out_f32) return ATOM_UNSUPPORTED;
+  if (m == 0) return ATOM_OK;
+  if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)partial) & 15) return ATOM_BAD_SHAPE;
+  SkinnyParams p{};
+  p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = bias; p.y = y; p.partial = partial;
+  p.m = m; p.k = k; p.out_f32 = out_f32;
+  p.n = gate ? 2 * n : n;
+  p.inter = gate ? n : 0;
+  p.tiles = skinny_tiles(n, gate);
+  skinny_plan(m, p.tiles, k, &p.splits, &p.kslice, &p.xk);
+  if (p.splits > 1 ? partial == nullptr : y == nullptr) return ATOM_BAD_SHAPE;
+  const long blocks = (long)p.tiles * p.splits;
+  if (blocks > 0x7fffffffL) return ATOM_TOO_LARGE;
+  const size_t lds = max((size_t)m * (p.xk * 2 + 16), (size_t)m * (kSkinnyRows + 1) * 4);
+  const int mt = (m + 15) / 16;
+#define GO(MTV)                                                                                             \
+  do {                                                                                                      \
+    if (gate) hipLaunchKernelGGL((gemm_skinny_kernel<MTV, true>), dim3(blocks), dim3(256), lds, stream, p); \
+    else hipLaunchKernelGGL((gemm_skinny_kernel<MTV, false>), dim3(blocks), dim3(256), lds, stream, p);     \
+  } while (0)
+  switch (mt) {
+    case 1: GO(1); break;
+    case 2: GO(2); break;
+    case 3: GO(3); break;
+    default: GO(4); break;
+  }
+#undef GO
+  return launch_status();
+}
+
+// y[m, n] = sum of partial[s][m][n] over s (+ bias): for readers that cannot add the slices themselves.
+ATOM_EXPORT int atom_splitk_reduce(const float* partial, const float* bias, void* y, int m, int n, int splits,
+                                   int out_f32, hipStream_t stream) {
+  if (m < 0 || n <= 0 || splits < 1) return ATOM_BAD_SHAPE;
+  const size_t total = (size_t)m * n;
+  if (total == 0) return ATOM_OK;
+  const size_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
+  if (out_f32) hipLaunchKernelGGL(splitk_reduce_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, partial,
+                                  bias, (float*)y, total, n, splits);
+  else hipLaunchKernelGGL(splitk_reduce_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, partial, bias,
+                          (bf16_t*)y, total, n, splits);
+  return launch_status();
+}

@@ -60,6 +60,34 @@ class AttentionMeta:
     rows_per_tile: int = 16
 
 
+class DeferredSum:
+    """A matrix product that is still a sum of slices: ``partial`` float32 [splits, rows, width], plus an
+    optional bias over the width.  The skinny product leaves its result like this when it cuts K; the
+    kernel that reads it next (norm, rotation, SiLU-mul) adds the slices in slice order while it reads.
+    ``dtype`` is the type the product has once it is a tensor (``HipKernels.materialize``)."""
+
+    def __init__(self, partial: torch.Tensor, bias: torch.Tensor | None, dtype: torch.dtype):
+        self.partial = partial
+        self.bias = bias
+        self.dtype = dtype
+
+    @property
+    def shape(self):
+        return self.partial.shape[1:]
+
+    @property
+    def device(self):
+        return self.partial.device
+
+    @property
+    def splits(self) -> int:
+        return self.partial.shape[0]
+
+    @property
+    def stride(self) -> int:
+        return self.partial.shape[1] * self.partial.shape[2]
+
+
 def _ptr(t: torch.Tensor | None):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else None
 
@@ -81,10 +109,12 @@ class HipKernels:
             raise KernelError(f"could not load the kernel library {path}: {e}") from e
         self.path = path
         for fn in ("atom_embedding", "atom_rmsnorm", "atom_silu_mul", "atom_qk_norm_rope_kv_write",
+                   "atom_gemm_skinny", "atom_gemm_skinny_splits", "atom_gemm_skinny_supports", "atom_splitk_reduce",
                    "atom_paged_attention_generic", "atom_gemm_f32", "atom_sample", "atom_exponential_noise",
                    "atom_attention_mfma_supports", "atom_attention_decode", "atom_attention_prefill"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
+        self.use_skinny_gemm = True    # bfloat16 products of at most 64 rows run this library's own kernel
         self.use_mfma_attention = True
         self._ws: dict[str, torch.Tensor] = {}
         self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
@@ -139,6 +169,26 @@ class HipKernels:
         except KeyError:
             raise KernelError(f"element type {t.dtype} is not supported (float32 and bfloat16 are)") from None
 
+    def _sum_args(self, x):
+        """The four trailing arguments that say whether an input is a tensor or a sum of slices."""
+        if isinstance(x, DeferredSum):
+            self._check("slices", x.partial, torch.float32)
+            if x.bias is not None:
+                self._check("bias of the slices", x.bias, torch.float32, (x.shape[1],))
+            return _ptr(x.partial), x.splits, ctypes.c_long(x.stride), _ptr(x.bias)
+        return None, 0, ctypes.c_long(0), None
+
+    def materialize(self, x):
+        """A tensor from what may still be a sum of slices."""
+        if not isinstance(x, DeferredSum):
+            return x
+        rows, width = x.shape
+        y = torch.empty((rows, width), dtype=x.dtype, device=x.device)
+        self._done("splitk_reduce", self.lib.atom_splitk_reduce(
+            _ptr(x.partial), _ptr(x.bias), _ptr(y), rows, width, x.splits, int(x.dtype == torch.float32),
+            self._stream()))
+        return y
+
     # ------------------------------------------------------------------ kernels
 
     def embedding(self, table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -158,7 +208,9 @@ class HipKernels:
         rows are normed (into out[0..len(rows))) and the residual is not written."""
         width = x.shape[-1]
         code = {"plain": 0, "init": 1, "add": 2}[mode]
-        self._check("norm input", x, (torch.float32, torch.bfloat16), (None, width))
+        deferred = isinstance(x, DeferredSum)
+        if not deferred:
+            self._check("norm input", x, (torch.float32, torch.bfloat16), (None, width))
         self._check("norm weight", weight, torch.float32, (width,))
         n_out = rows.numel() if rows is not None else x.shape[0]
         self._check("norm out", out, x.dtype, (n_out, width))
@@ -169,18 +221,20 @@ class HipKernels:
         if rows is not None:
             self._check("norm rows", rows, torch.int32, (n_out,))
         self._done("rmsnorm", self.lib.atom_rmsnorm(
-            _ptr(x), _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows), self._code(x), n_out, width,
-            ctypes.c_float(eps), code, self._stream()))
+            None if deferred else _ptr(x), _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows), self._code(out),
+            n_out, width, ctypes.c_float(eps), code, *self._sum_args(x), self._stream()))
         return out
 
     def silu_mul(self, x, out):
         rows, two = x.shape
         if two % 2:
             raise KernelError("silu_mul: the input width must be even (gate | up)")
-        self._check("silu_mul input", x, (torch.float32, torch.bfloat16))
+        deferred = isinstance(x, DeferredSum)
+        if not deferred:
+            self._check("silu_mul input", x, (torch.float32, torch.bfloat16))
         self._check("silu_mul out", out, x.dtype, (rows, two // 2))
-        self._done("silu_mul", self.lib.atom_silu_mul(_ptr(x), _ptr(out), self._code(x), rows, two // 2,
-                                                      self._stream()))
+        self._done("silu_mul", self.lib.atom_silu_mul(None if deferred else _ptr(x), _ptr(out), self._code(out), rows,
+                                                      two // 2, *self._sum_args(x), self._stream()))
         return out
 
     def qk_norm_rope_kv_write(self, qkv, q_out, k_cache, v_cache, q_weight, k_weight, cos, sin, positions,
@@ -188,7 +242,13 @@ class HipKernels:
                               page_size: int, eps: float, write_kv: bool = True):
         tokens = qkv.shape[0]
         dt = qkv.dtype
-        self._check("qkv", qkv, (torch.float32, torch.bfloat16), (tokens, (num_heads + 2 * num_kv_heads) * head_dim))
+        deferred = isinstance(qkv, DeferredSum)
+        if deferred:
+            if tuple(qkv.shape) != (tokens, (num_heads + 2 * num_kv_heads) * head_dim):
+                raise KernelError(f"qkv: shape {tuple(qkv.shape)} does not fit the heads")
+        else:
+            self._check("qkv", qkv, (torch.float32, torch.bfloat16),
+                        (tokens, (num_heads + 2 * num_kv_heads) * head_dim))
         self._check("q out", q_out, dt, (tokens, num_heads, head_dim))
         if write_kv:
             self._check("key pages", k_cache, dt, (None, num_kv_heads, page_size, head_dim))
@@ -202,11 +262,11 @@ class HipKernels:
             self._check("sin table", sin, torch.float32, tuple(cos.shape))
             self._check("positions", positions, torch.int32, (tokens,))
         self._done("qk_norm_rope_kv_write", self.lib.atom_qk_norm_rope_kv_write(
-            _ptr(qkv), _ptr(q_out), _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None,
+            None if deferred else _ptr(qkv), _ptr(q_out), _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None,
             _ptr(q_weight), _ptr(k_weight), _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None,
-            _ptr(positions) if rotary_dim else None, _ptr(slots) if write_kv else None, self._code(qkv), tokens,
+            _ptr(positions) if rotary_dim else None, _ptr(slots) if write_kv else None, self._code(q_out), tokens,
             num_heads, num_kv_heads, head_dim, rotary_dim, page_size, ctypes.c_float(eps), int(bool(write_kv)),
-            self._stream()))
+            *self._sum_args(qkv), self._stream()))
         return q_out
 
     def _attention_mfma(self, q, k_cache, v_cache, out, meta, scale, window, parts=None):
@@ -269,10 +329,17 @@ class HipKernels:
             ctypes.c_float(scale), int(window or 0), self._stream()))
         return out
 
-    def linear(self, x, weight, bias=None, out_dtype=None):
-        """``x @ weight.T (+ bias)``.  bfloat16 operands go to the BLAS library, as the
-        reference's engine does for its matrix products; anything with a float32 operand
-        runs this library's own float32 kernel (plain FMA, no reduced-precision mode)."""
+    def _skinny(self, x, weight) -> bool:
+        m, k = x.shape
+        return bool(self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                    and self.lib.atom_gemm_skinny_supports(m, weight.shape[0], k))
+
+    def linear(self, x, weight, bias=None, out_dtype=None, defer: bool = False):
+        """``x @ weight.T (+ bias)``.  bfloat16 operands with at most 64 rows run this library's own
+        weight-streaming kernel; with more rows they go to the BLAS library, as the reference's engine
+        does for its matrix products; anything with a float32 operand runs this library's float32
+        kernel (plain FMA, no reduced-precision mode).  With ``defer`` the result may come back as a
+        ``DeferredSum`` for a kernel that adds the slices while it reads them."""
         m, k = x.shape
         n = weight.shape[0]
         self._check("linear input", x, (torch.float32, torch.bfloat16))
@@ -280,6 +347,19 @@ class HipKernels:
         out_dtype = out_dtype or x.dtype
         if bias is not None:
             self._check("linear bias", bias, torch.float32, (n,))
+        if m and self._skinny(x, weight):
+            splits = self.lib.atom_gemm_skinny_splits(m, n, k, 0)
+            if splits == 1:
+                y = torch.empty((m, n), dtype=out_dtype, device=x.device)
+                self._done("gemm_skinny", self.lib.atom_gemm_skinny(
+                    _ptr(x), _ptr(weight), _ptr(bias), _ptr(y), None, m, n, k, int(out_dtype == torch.float32), 0,
+                    self._stream()))
+                return y
+            partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+            self._done("gemm_skinny", self.lib.atom_gemm_skinny(
+                _ptr(x), _ptr(weight), None, None, _ptr(partial), m, n, k, 0, 0, self._stream()))
+            result = DeferredSum(partial, bias, out_dtype)
+            return result if defer else self.materialize(result)
         if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and self.allow_library_gemm:
             y = torch.nn.functional.linear(x, weight)
             if bias is not None:
@@ -290,6 +370,33 @@ class HipKernels:
             _ptr(x), self._code(x), _ptr(weight), self._code(weight), _ptr(bias), _ptr(y), self._code(y), m, n, k,
             self._stream()))
         return y
+
+    def linear_silu(self, x, weight, bias=None):
+        """``silu(x @ Wg.T + bg) * (x @ Wu.T + bu)`` for ``weight`` = gate rows then up rows: one kernel
+        where the skinny product does not cut K, else the product and SiLU-mul over its slices."""
+        m, k = x.shape
+        two = weight.shape[0]
+        if two % 2:
+            raise KernelError("linear_silu: the weight must hold as many gate rows as up rows")
+        inter = two // 2
+        if m and self._skinny(x, weight):
+            self._check("linear input", x, torch.bfloat16)
+            self._check("linear weight", weight, torch.bfloat16, (two, k))
+            if bias is not None:
+                self._check("linear bias", bias, torch.float32, (two,))
+            act = torch.empty((m, inter), dtype=x.dtype, device=x.device)
+            splits = self.lib.atom_gemm_skinny_splits(m, inter, k, 1)
+            if splits == 1:
+                self._done("gemm_skinny", self.lib.atom_gemm_skinny(
+                    _ptr(x), _ptr(weight), _ptr(bias), _ptr(act), None, m, inter, k, 0, 1, self._stream()))
+                return act
+            partial = torch.empty((splits, m, two), dtype=torch.float32, device=x.device)
+            self._done("gemm_skinny", self.lib.atom_gemm_skinny(
+                _ptr(x), _ptr(weight), None, None, _ptr(partial), m, inter, k, 0, 1, self._stream()))
+            return self.silu_mul(DeferredSum(partial, bias, x.dtype), act)
+        gate_up = self.linear(x, weight, bias)
+        act = torch.empty((m, inter), dtype=x.dtype, device=x.device)
+        return self.silu_mul(gate_up, act)
 
     def sample(self, logits, temperatures, out, top_ks=None, top_ps=None, noise=None, seeds=None, counters=None,
                eps: float = 1e-10):

@@ -86,5 +86,7 @@ class CausalLM(Part):
             hidden, residual = self.blocks[run.layer].forward(ctx, hidden, residual, cache)
         if want_rows is None or want_rows.numel() == 0:
             return None
+        if not self.final_norm.accepts_deferred:
+            hidden = ctx.ops.materialize(hidden)
         normed = self.final_norm.forward_rows(ctx, hidden, residual, want_rows)
         return self.head.forward(ctx, normed)

@@ -71,7 +71,7 @@ class GroupedQueryAttention(Mixer):
     def forward(self, ctx, x, cache):
         ops = ctx.ops
         tokens = x.shape[0]
-        qkv = ops.linear(x, self.params["qkv.weight"], self.p("qkv.bias"))
+        qkv = ops.linear(x, self.params["qkv.weight"], self.p("qkv.bias"), defer=True)
         q = torch.empty((tokens, self.num_heads, self.head_dim), dtype=x.dtype, device=x.device)
         meta = ctx.attention[cache.group]
         rope = self.rope
@@ -82,7 +82,8 @@ class GroupedQueryAttention(Mixer):
             rope.rotary_dim if rope else 0, meta.page_size, self.norm_eps, write_kv=cache.writes)
         out = torch.empty_like(q)
         ops.paged_attention(q, cache.k_cache, cache.v_cache, out, meta, self.scale, self.window)
-        return ops.linear(out.view(tokens, self.num_heads * self.head_dim), self.params["o.weight"], self.p("o.bias"))
+        return ops.linear(out.view(tokens, self.num_heads * self.head_dim), self.params["o.weight"], self.p("o.bias"),
+                          defer=True)
 
 
 MIXERS.register("attention", GroupedQueryAttention)

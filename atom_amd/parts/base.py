@@ -117,6 +117,11 @@ class StateNeed:
 
 
 class Norm(Part):
+    #: True when the norm hands ``x`` to ``ctx.ops.rmsnorm`` as it is: a mixer or feed-forward may return
+    #: a product that is still a sum of slices (``ops.linear(..., defer=True)``), which that kernel adds
+    #: while it reads.  Other norms get a tensor (the block calls ``ops.materialize`` first).
+    accepts_deferred = False
+
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 

@@ -27,8 +27,12 @@ class PreNormBlock(Block):
         return [self.mixer_norm, self._mixer, self.ffn_norm, self.ffn]
 
     def forward(self, ctx, hidden, residual, cache):
+        if not self.mixer_norm.accepts_deferred:
+            hidden = ctx.ops.materialize(hidden)
         hidden, residual = self.mixer_norm.forward_residual(ctx, hidden, residual)
         hidden = self._mixer.forward(ctx, hidden, cache)
+        if not self.ffn_norm.accepts_deferred:
+            hidden = ctx.ops.materialize(hidden)
         hidden, residual = self.ffn_norm.forward_residual(ctx, hidden, residual)
         hidden = self.ffn.forward(ctx, hidden)
         return hidden, residual

@@ -34,10 +34,9 @@ class GatedMLP(FeedForward):
 
     def forward(self, ctx, x):
         ops = ctx.ops
-        gate_up = ops.linear(x, self.params["gate_up.weight"], self.p("gate_up.bias"))
-        act = torch.empty((x.shape[0], self.intermediate_size), dtype=x.dtype, device=x.device)
-        ops.silu_mul(gate_up, act)
-        return ops.linear(act, self.params["down.weight"], self.p("down.bias"))
+        act = ops.linear_silu(x, self.params["gate_up.weight"], self.p("gate_up.bias"))
+        # the down product may come back as slices that the next norm adds while it reads them
+        return ops.linear(act, self.params["down.weight"], self.p("down.bias"), defer=True)
 
 
 FEED_FORWARDS.register("gated_mlp", GatedMLP)

@@ -9,6 +9,8 @@ from .base import NORMS, Norm, ParamSpec
 
 
 class RMSNorm(Norm):
+    accepts_deferred = True   # the kernel adds the slices of a product that is still a sum
+
     def __init__(self, size: int, eps: float, prefix: str = ""):
         super().__init__(prefix)
         self.size = size
@@ -18,13 +20,13 @@ class RMSNorm(Norm):
         return {"weight": ParamSpec.single("weight", (self.size,), kind="vector", init="one_plus_normal")}
 
     def forward(self, ctx, x):
-        out = torch.empty_like(x)
+        out = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
         return ctx.ops.rmsnorm(x, self.params["weight"], self.eps, out)
 
     def forward_residual(self, ctx, x, residual):
-        out = torch.empty_like(x)
+        out = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
         if residual is None:
-            residual = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+            residual = torch.empty(tuple(x.shape), dtype=torch.float32, device=x.device)
             ctx.ops.rmsnorm(x, self.params["weight"], self.eps, out, residual=residual, mode="init")
         else:
             ctx.ops.rmsnorm(x, self.params["weight"], self.eps, out, residual=residual, mode="add")

@@ -88,11 +88,17 @@ class PlainKernels:
             out[t] = o[0].to(out.dtype)
         return out
 
-    def linear(self, x, weight, bias=None, out_dtype=None):
+    def linear(self, x, weight, bias=None, out_dtype=None, defer=False):
         y = x.to(WIDE) @ weight.to(WIDE).T
         if bias is not None:
             y = y + bias.to(WIDE)
         return y.to(out_dtype or x.dtype)
+
+    def linear_silu(self, x, weight, bias=None):
+        return silu_and_mul(self.linear(x, weight, bias, out_dtype=WIDE)).to(x.dtype)
+
+    def materialize(self, x):
+        return x
 
     def exponential_noise(self, seeds, counters, vocab):
         rows = []

@@ -359,3 +359,115 @@ def test_kernels_refuse_what_they_cannot_take():
     with pytest.raises(KernelError):
         ops.embedding(torch.zeros((10, 8), device=DEV, dtype=torch.float16), torch.zeros(2, dtype=torch.int32, device=DEV),
                       torch.zeros((2, 8), device=DEV))
+
+
+# ------------------------------------------------------------------ the skinny matrix product
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 311, 136), (8, 4096, 4096), (16, 517, 200), (17, 1000, 520), (33, 96, 2056),
+                                   (64, 640, 1032), (5, 64, 8), (3, 6144, 4096), (7, 130, 12288)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_skinny_gemm(m, n, k, out_dtype):
+    ops = gpu_ops()
+    x = rnd((m, k), torch.bfloat16, 40, 1.0)
+    w = rnd((n, k), torch.bfloat16, 41, 0.05)
+    b = rnd((n,), torch.float32, 42, 0.5)
+    assert ops.lib.atom_gemm_skinny_supports(m, n, k)
+    want = x.double() @ w.double().T + b.double()
+    y = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), out_dtype=out_dtype)
+    assert y.dtype == out_dtype
+    close(y, want, out_dtype if out_dtype == torch.bfloat16 else torch.bfloat16, scale=float(want.abs().max()))
+    if out_dtype == torch.float32:   # float32 out keeps the float32 accumulation: far closer than a bfloat16 ulp
+        assert float((y.cpu().double() - want).abs().max()) <= 1e-4 * float(want.abs().max())
+    # a row's result does not depend on the rows beside it
+    if m > 1:
+        alone = ops.linear(x[m - 1:].to(DEV).contiguous(), w.to(DEV), b.to(DEV), out_dtype=out_dtype)
+        assert torch.equal(alone[0], y[m - 1])
+
+
+def test_skinny_gemm_is_what_runs():
+    """At most 64 bfloat16 rows take the engine's own kernel, not the library."""
+    ops = gpu_ops()
+    x = rnd((8, 512), torch.bfloat16, 1).to(DEV)
+    w = rnd((256, 512), torch.bfloat16, 2, 0.05).to(DEV)
+    ops.allow_library_gemm = False
+    try:
+        y = ops.linear(x, w)
+    finally:
+        ops.allow_library_gemm = True
+    close(y, x.cpu().double() @ w.cpu().double().T, torch.bfloat16)
+
+
+@pytest.mark.parametrize("m,inter,k", [(1, 200, 136), (8, 12288, 4096), (20, 333, 264), (64, 160, 96)])
+def test_skinny_gemm_silu_gate(m, inter, k):
+    ops = gpu_ops()
+    x = rnd((m, k), torch.bfloat16, 50, 1.0)
+    w = rnd((2 * inter, k), torch.bfloat16, 51, 0.05)
+    b = rnd((2 * inter,), torch.float32, 52, 0.3)
+    gu = x.double() @ w.double().T + b.double()
+    want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    act = ops.linear_silu(x.to(DEV), w.to(DEV), b.to(DEV))
+    close(act, want, torch.bfloat16)
+    swapped = torch.nn.functional.silu(gu[:, inter:]) * gu[:, :inter]
+    assert float((swapped - want).abs().max()) > 0.05 * float(want.abs().max())
+
+
+def _deferred(ops, m, n, k, seed, bias=True):
+    """A product as the skinny kernel leaves it when it cuts K, and the same as float64."""
+    from atom_amd.kernels.hip import DeferredSum
+
+    x = rnd((m, k), torch.bfloat16, seed, 1.0)
+    w = rnd((n, k), torch.bfloat16, seed + 1, 0.05)
+    b = rnd((n,), torch.float32, seed + 2, 0.3) if bias else None
+    got = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV) if bias else None, defer=True)
+    assert isinstance(got, DeferredSum) and got.splits > 1, "this shape was chosen so that K is cut"
+    want = x.double() @ w.double().T + (b.double() if bias else 0)
+    return got, want
+
+
+def test_deferred_sum_readers():
+    """Norm, rotation and SiLU-mul read a product that is still a sum of slices."""
+    ops = gpu_ops()
+    # norm with the residual sum
+    d, want = _deferred(ops, 6, 256, 4096, 60)
+    wn = 1 + rnd((256,), torch.float32, 63, 0.2)
+    res = rnd((6, 256), torch.float32, 64)
+    out = torch.empty((6, 256), dtype=torch.bfloat16, device=DEV)
+    res_gpu = res.to(DEV)
+    ops.rmsnorm(d, wn.to(DEV), 1e-5, out, residual=res_gpu, mode="add")
+    summed = want + res.double()
+    norm = summed * torch.rsqrt((summed ** 2).mean(-1, keepdim=True) + 1e-5) * wn.double()
+    close(out, norm, torch.bfloat16)
+    close(res_gpu, summed, torch.float32, scale=float(summed.abs().max()) * 50)   # sums of bfloat16 products
+    # norm at chosen rows, width that is no multiple of 8 pieces per thread
+    rows = torch.tensor([5, 0], dtype=torch.int32, device=DEV)
+    out2 = torch.empty((2, 256), dtype=torch.bfloat16, device=DEV)
+    ops.rmsnorm(d, wn.to(DEV), 1e-5, out2, residual=res.to(DEV), mode="add", rows=rows)
+    close(out2, norm[[5, 0]], torch.bfloat16)
+    # materialize
+    close(ops.materialize(d), want, torch.bfloat16)
+    # SiLU-mul
+    d, want = _deferred(ops, 4, 2 * 136, 2048, 70)
+    act = torch.empty((4, 136), dtype=torch.bfloat16, device=DEV)
+    ops.silu_mul(d, act)
+    close(act, torch.nn.functional.silu(want[:, :136]) * want[:, 136:], torch.bfloat16)
+    # rotation and cache write: against the same kernel fed the tensor
+    hq, hkv, hd, page = 4, 2, 32, 16
+    d, want = _deferred(ops, 5, (hq + 2 * hkv) * hd, 4096, 80)
+    qkv = want.to(torch.bfloat16).to(DEV)
+    pos = torch.tensor([3, 9, 0, 17, 30], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([3, 9, 16, -1, 46], dtype=torch.int32, device=DEV)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))
+    ang = torch.arange(64).float()[:, None] * inv[None, :]
+    cos, sin = ang.cos().to(DEV), ang.sin().to(DEV)
+    wq = (1 + rnd((hd,), torch.float32, 83, 0.2)).to(DEV)
+    wk = (1 + rnd((hd,), torch.float32, 84, 0.2)).to(DEV)
+    outs = []
+    for src in (d, qkv):
+        q = torch.zeros((5, hq, hd), dtype=torch.bfloat16, device=DEV)
+        kc = torch.zeros((4, hkv, page, hd), dtype=torch.bfloat16, device=DEV)
+        vc = torch.zeros((4, hkv, hd, page), dtype=torch.bfloat16, device=DEV)
+        ops.qk_norm_rope_kv_write(src, q, kc, vc, wq, wk, cos, sin, pos, slots, hq, hkv, hd, hd, page, 1e-6)
+        outs.append((q, kc, vc))
+    for a, b in zip(*outs):
+        close(a, b.double(), torch.bfloat16, scale=float(b.abs().max()) * 2)
