@@ -16,6 +16,11 @@
 // or atom_splitk_reduce.  The sum has one fixed order, so a row's result does not
 // depend on its batch.
 //
+// A wide product (256 row tiles or more: the gate/up and head products) runs with sixteen waves a
+// block instead: four groups of four waves share the block's rows and x slice and each take a
+// quarter of its K, and their sums are added through LDS in group order.  That puts enough loads
+// in flight without cutting K between blocks, so the epilogue can be applied at once.
+//
 // Epilogues when K is not cut: plain (bias optional, bfloat16 or float32 out), or
 // SiLU-gate: w holds `inter` gate rows then `inter` up rows, a block owns 32 columns of
 // each, and writes silu(gate) * up [M, inter].
@@ -35,18 +40,24 @@ struct SkinnyParams {
   int m, n, k, inter, out_f32, splits, tiles, kslice, xk;
 };
 
+struct SkinnyPlan {
+  int splits, kslice, xk, kgroups;
+};
+
 constexpr int kSkinnyRows = 64;    // rows of w per block
 constexpr int kSkinnyChunk = 256;  // k elements per chunk
 constexpr int kSkinnyU = kSkinnyChunk / 32;
 constexpr int kSkinnyLds = 64 * 1024;
 
-template <int MT, bool GATE>
-__global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
+template <int MT, bool GATE, int KG>
+__global__ void __launch_bounds__(256 * KG) gemm_skinny_kernel(SkinnyParams p) {
   constexpr int U = kSkinnyU;
-  extern __shared__ __attribute__((aligned(16))) char smem[];   // x slice; later the float32 tile
+  constexpr int THREADS = 256 * KG;
+  extern __shared__ __attribute__((aligned(16))) char smem[];   // x slice; later the float32 tiles
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
-  const int wave = tid / kWave;
+  const int wave = (tid / kWave) & 3;    // which 16 of the block's 64 rows
+  const int kgroup = tid / (4 * kWave);  // which part of the block's K slice
   const int r16 = lane & 15;
   const int g = lane >> 4;
   const int k = p.k;
@@ -54,6 +65,10 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
   const int split = blockIdx.x - tile * p.splits;
   const int k_begin = split * p.kslice;
   const int k_end = min(k, k_begin + p.kslice);
+  // this wave's part of the slice: whole chunks
+  const int sub = ((p.kslice / KG + kSkinnyChunk - 1) / kSkinnyChunk) * kSkinnyChunk;
+  const int kw_begin = k_begin + kgroup * sub;
+  const int kw_end = min(k_end, kw_begin + sub);
   const int xrow_bytes = p.xk * 2 + 16;   // 16 bytes of padding: rows start 4 banks apart
 
   // the row of w this lane streams, and the output column it stands for
@@ -82,13 +97,14 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
       a_next[u] = (kk + 8 * g < k) ? *reinterpret_cast<const bf16x8*>(wp + kk) : zero;
     }
   };
-  if (k_begin < k_end) load_a(k_begin);
+  const int nch = kw_begin < kw_end ? (kw_end - kw_begin + kSkinnyChunk - 1) / kSkinnyChunk : 0;
+  if (nch) load_a(kw_begin);
 
   for (int x0 = k_begin; x0 < k_end; x0 += p.xk) {
     const int x1 = min(k_end, x0 + p.xk);
     const int pieces = (x1 - x0 + 7) / 8;    // 16-byte pieces per row
     if (x0 != k_begin) __syncthreads();      // the previous slice of x has been read
-    for (int q = tid; q < p.m * pieces; q += 256) {
+    for (int q = tid; q < p.m * pieces; q += THREADS) {
       const int row = q / pieces, piece = q - row * pieces;
       const int kk = x0 + 8 * piece;
       const bf16x8 v = kk < k ? *reinterpret_cast<const bf16x8*>(p.x + (size_t)row * k + kk) : zero;
@@ -96,16 +112,16 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
     }
     // a chunk that reaches beyond K reads pieces the loop above did not write: zero them
     const int padded = ((x1 - x0 + kSkinnyChunk - 1) / kSkinnyChunk) * (kSkinnyChunk / 8);
-    for (int q = tid; q < p.m * (padded - pieces); q += 256) {
+    for (int q = tid; q < p.m * (padded - pieces); q += THREADS) {
       const int row = q / (padded - pieces), piece = pieces + q - row * (padded - pieces);
       *reinterpret_cast<bf16x8*>(smem + row * xrow_bytes + piece * 16) = zero;
     }
     __syncthreads();
-    for (int kc = x0; kc < x1; kc += kSkinnyChunk) {
+    for (int kc = max(x0, kw_begin); kc < min(x1, kw_end); kc += kSkinnyChunk) {
       bf16x8 a[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) a[u] = a_next[u];
-      if (kc + kSkinnyChunk < k_end) load_a(kc + kSkinnyChunk);
+      if (kc + kSkinnyChunk < kw_end) load_a(kc + kSkinnyChunk);
       const char* xb = smem + (kc - x0) * 2;
 #pragma unroll
       for (int u = 0; u < U; ++u)
@@ -117,22 +133,35 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
     }
   }
 
-  // ---- the block's float32 tile [m][64] through LDS: lane holds rows m = 16 t + r16, columns 16 wave + 4 g + i
+  // ---- the block's float32 tile [m][64] through LDS, one per K group, added in group order:
+  //      lane holds rows m = 16 t + r16, columns 16 wave + 4 g + i
   __syncthreads();
-  float* tile_f = reinterpret_cast<float*>(smem);   // [m][65]
+  float* tile_f = reinterpret_cast<float*>(smem);   // [KG][m][65], then [m][65]
+  const int tile_floats = p.m * (kSkinnyRows + 1);
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = 16 * t + r16;
     if (m < p.m) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) tile_f[m * (kSkinnyRows + 1) + 16 * wave + 4 * g + i] = acc[t][i];
+      for (int i = 0; i < 4; ++i)
+        tile_f[kgroup * tile_floats + m * (kSkinnyRows + 1) + 16 * wave + 4 * g + i] = acc[t][i];
     }
   }
   __syncthreads();
+  if (KG > 1) {
+    for (int item = tid; item < p.m * kSkinnyRows; item += THREADS) {
+      const int at = (item >> 6) * (kSkinnyRows + 1) + (item & 63);
+      float v = tile_f[at];
+#pragma unroll
+      for (int kg = 1; kg < KG; ++kg) v += tile_f[kg * tile_floats + at];
+      tile_f[at] = v;
+    }
+    __syncthreads();
+  }
 
   if (p.splits > 1) {
     float* mine = p.partial + (size_t)split * p.m * p.n;
-    for (int item = tid; item < p.m * kSkinnyRows; item += 256) {
+    for (int item = tid; item < p.m * kSkinnyRows; item += THREADS) {
       const int m = item >> 6, c = item & 63;
       int col;
       if (GATE) {
@@ -148,7 +177,7 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
     return;
   }
   if (GATE) {
-    for (int item = tid; item < p.m * 32; item += 256) {
+    for (int item = tid; item < p.m * 32; item += THREADS) {
       const int m = item >> 5, c = item & 31;
       const int col = tile * 32 + c;
       if (col >= p.inter) continue;
@@ -161,7 +190,7 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
       reinterpret_cast<bf16_t*>(p.y)[(size_t)m * p.inter + col] = from_f32<bf16_t>(gv / (1.f + expf(-gv)) * uv);
     }
   } else {
-    for (int item = tid; item < p.m * kSkinnyRows; item += 256) {
+    for (int item = tid; item < p.m * kSkinnyRows; item += THREADS) {
       const int m = item >> 6, c = item & 63;
       const int col = tile * kSkinnyRows + c;
       if (col >= p.n) continue;
@@ -186,17 +215,32 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, const fl
 
 static int skinny_tiles(int n, int gate) { return gate ? (n + 31) / 32 : (n + kSkinnyRows - 1) / kSkinnyRows; }
 
-// How K is cut: enough blocks to keep about a thousand in flight, slices a multiple of 512.
-static void skinny_plan(int m, int tiles, int k, int* splits, int* kslice, int* xk) {
+// How K is cut between blocks (slices a multiple of 512) and inside a block.
+static SkinnyPlan skinny_plan(int m, int tiles, int k) {
+  SkinnyPlan plan{};
   const int units = (k + 511) / 512;
+  if (tiles >= 256) {
+    // wide: sixteen waves a block, four K groups; the block's whole x slice sits in LDS, two blocks a CU
+    // where 80 KB hold it, else one
+    plan.kgroups = 4;
+    int cap = ((80 * 1024 / m - 16) / 2) / 1024 * 1024;
+    if (cap < 1024) cap = ((144 * 1024 / m - 16) / 2) / 1024 * 1024;   // m <= 64: at least 1024
+    plan.kslice = min(units * 512, cap);
+    plan.splits = (k + plan.kslice - 1) / plan.kslice;
+    plan.xk = ((plan.kslice + kSkinnyChunk - 1) / kSkinnyChunk) * kSkinnyChunk;
+    return plan;
+  }
+  // narrow: four waves a block and enough slices to keep about a thousand blocks in flight
+  plan.kgroups = 1;
   int s = (1024 + tiles - 1) / tiles;
   s = max(1, min(s, min(units, 32)));
   const int per = (units + s - 1) / s;           // units of 512 per slice
-  *kslice = per * 512;
-  *splits = (units + per - 1) / per;
+  plan.kslice = per * 512;
+  plan.splits = (units + per - 1) / per;
   int cap = (kSkinnyLds - 64) / m / 2 - 8;       // k elements of one row of x that fit
   cap = max(kSkinnyChunk, cap / kSkinnyChunk * kSkinnyChunk);
-  *xk = min(*kslice, cap);
+  plan.xk = min(plan.kslice, cap);
+  return plan;
 }
 
 // 1 if the skinny kernel takes this product.
@@ -206,9 +250,7 @@ ATOM_EXPORT int atom_gemm_skinny_supports(int m, int n, int k) {
 
 // Into how many slices atom_gemm_skinny cuts K for this product (1: it writes y itself).
 ATOM_EXPORT int atom_gemm_skinny_splits(int m, int n, int k, int gate) {
-  int splits, kslice, xk;
-  skinny_plan(max(m, 1), skinny_tiles(n, gate), k, &splits, &kslice, &xk);
-  return splits;
+  return skinny_plan(max(m, 1), skinny_tiles(n, gate), k).splits;
 }
 
 // gate == 0: x w^T, n columns.  gate == 1: w is [2 n, k] (n gate rows, then n up rows).
@@ -228,16 +270,34 @@ ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias
   p.n = gate ? 2 * n : n;
   p.inter = gate ? n : 0;
   p.tiles = skinny_tiles(n, gate);
-  skinny_plan(m, p.tiles, k, &p.splits, &p.kslice, &p.xk);
+  const SkinnyPlan plan = skinny_plan(m, p.tiles, k);
+  p.splits = plan.splits; p.kslice = plan.kslice; p.xk = plan.xk;
   if (p.splits > 1 ? partial == nullptr : y == nullptr) return ATOM_BAD_SHAPE;
   const long blocks = (long)p.tiles * p.splits;
   if (blocks > 0x7fffffffL) return ATOM_TOO_LARGE;
-  const size_t lds = max((size_t)m * (p.xk * 2 + 16), (size_t)m * (kSkinnyRows + 1) * 4);
+  const size_t lds = max((size_t)m * (p.xk * 2 + 16), (size_t)plan.kgroups * m * (kSkinnyRows + 1) * 4);
   const int mt = (m + 15) / 16;
-#define GO(MTV)                                                                                             \
-  do {                                                                                                      \
-    if (gate) hipLaunchKernelGGL((gemm_skinny_kernel<MTV, true>), dim3(blocks), dim3(256), lds, stream, p); \
-    else hipLaunchKernelGGL((gemm_skinny_kernel<MTV, false>), dim3(blocks), dim3(256), lds, stream, p);     \
+  const bool wide = plan.kgroups == 4;
+  // the wide kernels may need more LDS than a launch gets by default: allow it once per kernel
+#define GO_ONE(MTV, G, KGV)                                                                                   \
+  do {                                                                                                        \
+    if (KGV > 1) {                                                                                            \
+      static bool allowed = false;                                                                            \
+      if (!allowed) {                                                                                         \
+        if (hipFuncSetAttribute((const void*)gemm_skinny_kernel<MTV, G, KGV>,                                 \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)        \
+          return ATOM_LAUNCH_FAILED;                                                                          \
+        allowed = true;                                                                                       \
+      }                                                                                                       \
+    }                                                                                                         \
+    hipLaunchKernelGGL((gemm_skinny_kernel<MTV, G, KGV>), dim3(blocks), dim3(256 * KGV), lds, stream, p);     \
+  } while (0)
+#define GO(MTV)                                  \
+  do {                                           \
+    if (gate && wide) GO_ONE(MTV, true, 4);      \
+    else if (gate) GO_ONE(MTV, true, 1);         \
+    else if (wide) GO_ONE(MTV, false, 4);        \
+    else GO_ONE(MTV, false, 1);                  \
   } while (0)
   switch (mt) {
     case 1: GO(1); break;
@@ -246,6 +306,7 @@ ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias
     default: GO(4); break;
   }
 #undef GO
+#undef GO_ONE
   return launch_status();
 }
 

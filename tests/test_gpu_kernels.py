@@ -418,7 +418,8 @@ def test_kernels_refuse_what_they_cannot_take():
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 311, 136), (8, 4096, 4096), (16, 517, 200), (17, 1000, 520), (33, 96, 2056),
-                                   (64, 640, 1032), (5, 64, 8), (3, 6144, 4096), (7, 130, 12288)])
+                                   (64, 640, 1032), (5, 64, 8), (3, 6144, 4096), (7, 130, 12288),
+                                   (3, 16400, 520), (40, 16390, 1032), (8, 20000, 4096), (64, 16384, 2056)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_skinny_gemm(m, n, k, out_dtype):
     ops = gpu_ops()
@@ -432,10 +433,14 @@ def test_skinny_gemm(m, n, k, out_dtype):
     close(y, want, out_dtype if out_dtype == torch.bfloat16 else torch.bfloat16, scale=float(want.abs().max()))
     if out_dtype == torch.float32:   # float32 out keeps the float32 accumulation: far closer than a bfloat16 ulp
         assert float((y.cpu().double() - want).abs().max()) <= 1e-4 * float(want.abs().max())
-    # a row's result does not depend on the rows beside it
+    # a row's result does not depend on the rows beside it: to the bit while K is cut the same way (narrow
+    # products), within rounding for the wide ones, whose blocks take what K their x slice leaves room for
     if m > 1:
         alone = ops.linear(x[m - 1:].to(DEV).contiguous(), w.to(DEV), b.to(DEV), out_dtype=out_dtype)
-        assert torch.equal(alone[0], y[m - 1])
+        if n < 256 * 64:
+            assert torch.equal(alone[0], y[m - 1])
+        else:
+            close(alone[0], y[m - 1].double(), torch.bfloat16)
 
 
 def test_skinny_gemm_is_what_runs():
@@ -451,7 +456,8 @@ def test_skinny_gemm_is_what_runs():
     close(y, x.cpu().double() @ w.cpu().double().T, torch.bfloat16)
 
 
-@pytest.mark.parametrize("m,inter,k", [(1, 200, 136), (8, 12288, 4096), (20, 333, 264), (64, 160, 96)])
+@pytest.mark.parametrize("m,inter,k", [(1, 200, 136), (8, 12288, 4096), (20, 333, 264), (64, 160, 96),
+                                       (33, 8200, 1032), (64, 8192, 4096)])
 def test_skinny_gemm_silu_gate(m, inter, k):
     ops = gpu_ops()
     x = rnd((m, k), torch.bfloat16, 50, 1.0)
