@@ -117,7 +117,10 @@ class HipKernels:
                    "atom_attention_prefill_tile_rows"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
-        self.use_skinny_gemm = True    # bfloat16 products of at most 64 rows run this library's own kernel
+        # bfloat16 products of few rows run this library's own weight-streaming kernel.  It takes up to 64
+        # rows; beyond 16 (one matrix-core tile of rows) the BLAS library's kernels are faster on gfx950.
+        self.use_skinny_gemm = True
+        self.skinny_max_rows = 16
         self.use_mfma_attention = True
         self.use_tiled_prefill = True
         self._ws: dict[str, torch.Tensor] = {}
@@ -340,8 +343,8 @@ class HipKernels:
 
     def _skinny(self, x, weight) -> bool:
         m, k = x.shape
-        return bool(self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                    and self.lib.atom_gemm_skinny_supports(m, weight.shape[0], k))
+        return bool(self.use_skinny_gemm and m <= self.skinny_max_rows and x.dtype == torch.bfloat16
+                    and weight.dtype == torch.bfloat16 and self.lib.atom_gemm_skinny_supports(m, weight.shape[0], k))
 
     def linear(self, x, weight, bias=None, out_dtype=None, defer: bool = False):
         """``x @ weight.T (+ bias)``.  bfloat16 operands with at most 64 rows run this library's own

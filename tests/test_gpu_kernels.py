@@ -417,16 +417,27 @@ def test_kernels_refuse_what_they_cannot_take():
 # ------------------------------------------------------------------ the skinny matrix product
 
 
+@pytest.fixture
+def all_rows():
+    """The skinny kernel for every row count it takes (the engine hands it at most 16 rows)."""
+    ops = gpu_ops()
+    before = ops.skinny_max_rows
+    ops.skinny_max_rows = 64
+    yield ops
+    ops.skinny_max_rows = before
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 311, 136), (8, 4096, 4096), (16, 517, 200), (17, 1000, 520), (33, 96, 2056),
                                    (64, 640, 1032), (5, 64, 8), (3, 6144, 4096), (7, 130, 12288),
                                    (3, 16400, 520), (40, 16390, 1032), (8, 20000, 4096), (64, 16384, 2056)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-def test_skinny_gemm(m, n, k, out_dtype):
-    ops = gpu_ops()
+def test_skinny_gemm(m, n, k, out_dtype, all_rows):
+    ops = all_rows
     x = rnd((m, k), torch.bfloat16, 40, 1.0)
     w = rnd((n, k), torch.bfloat16, 41, 0.05)
     b = rnd((n,), torch.float32, 42, 0.5)
     assert ops.lib.atom_gemm_skinny_supports(m, n, k)
+    assert ops._skinny(x.to(DEV), w.to(DEV)), "this product must take the skinny kernel"
     want = x.double() @ w.double().T + b.double()
     y = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), out_dtype=out_dtype)
     assert y.dtype == out_dtype
@@ -458,8 +469,8 @@ def test_skinny_gemm_is_what_runs():
 
 @pytest.mark.parametrize("m,inter,k", [(1, 200, 136), (8, 12288, 4096), (20, 333, 264), (64, 160, 96),
                                        (33, 8200, 1032), (64, 8192, 4096)])
-def test_skinny_gemm_silu_gate(m, inter, k):
-    ops = gpu_ops()
+def test_skinny_gemm_silu_gate(m, inter, k, all_rows):
+    ops = all_rows
     x = rnd((m, k), torch.bfloat16, 50, 1.0)
     w = rnd((2 * inter, k), torch.bfloat16, 51, 0.05)
     b = rnd((2 * inter,), torch.float32, 52, 0.3)
