@@ -336,26 +336,25 @@ static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
 //
 // A block of four waves owns a tile of query tokens of GH query heads that share a KV head
 // (GH = 4, 2 or 1, a divisor of the group size): wave w has head (w % GH) and the 32 tokens
-// number (w / GH) of the tile, so a block covers 32 * 4 / GH tokens.  Keys are walked 32 at a
-// time; the block loads each K tile (32 keys x D) and V^T tile (D x 32 keys) once, through
+// number (w / GH) of the tile, so a block covers 32 * 4 / GH tokens.  Keys are walked TK (32) at a
+// time; the block loads each K tile (TK keys x D) and V^T tile (D x TK keys) once, through
 // registers (the next tile's loads are in flight while this one is multiplied) into LDS, where all
 // four waves read them as matrix-core operands.  Products, softmax and layouts are those of the
-// kernel above, with both products on v_mfma_f32_16x16x32_bf16: the 32 keys of a tile are the k
-// dimension of the second product, in the order (4 g + i, 16 + 4 g + i) that the first product
+// kernel above, with both products on v_mfma_f32_16x16x32_bf16: 32 keys of a tile are the k
+// dimension of one step of the second product, in the order (4 g + i, 16 + 4 g + i) that the first product
 // leaves them in a lane.
 //
 // Needs D % 64 == 0 and page_size % 8 == 0.
-constexpr int kTileKeys = 32;
-
-template <int D, int GH>
+template <int D, int GH, int TK>
 __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams p) {
   constexpr int KCH = D / 32;
   constexpr int DT = D / 16;
   constexpr int RT = 2;
+  constexpr int KB = TK / 16;            // blocks of 16 keys in a tile
   constexpr int KSTR = D + 8;            // LDS row of a key, in elements: rows start 4 banks apart
-  constexpr int VSTR = kTileKeys + 4;    // LDS row of V^T (one d), in elements
-  constexpr int PT = D / 64;             // 16-byte pieces of each tile that a thread moves
-  __shared__ __attribute__((aligned(16))) bf16_t ks[kTileKeys * KSTR];
+  constexpr int VSTR = TK + 4;           // LDS row of V^T (one d), in elements
+  constexpr int PT = D * TK / 8 / 256;   // 16-byte pieces of each tile that a thread moves
+  __shared__ __attribute__((aligned(16))) bf16_t ks[TK * KSTR];
   __shared__ __attribute__((aligned(16))) bf16_t vs[D * VSTR];
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -383,7 +382,7 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
   const int ke = pos_block0 + block_rows;           // one past the last key any row of the block sees
   const int my_ke = pos0 + nrows;
   int kb = 0;
-  if (p.window > 0 && pos_block0 - p.window + 1 > 0) kb = (pos_block0 - p.window + 1) & ~(kTileKeys - 1);
+  if (p.window > 0 && pos_block0 - p.window + 1 > 0) kb = (pos_block0 - p.window + 1) & ~(TK - 1);
   const int* table = p.block_tables + (size_t)seq * p.max_blocks;
 
   // ---- this wave's queries
@@ -414,7 +413,7 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
   }
 
   // ---- moving a tile: piece q of K is (key q / (D/8), 8 elements at (q % (D/8)) * 8);
-  //      piece q of V^T is (d = q / 4, the 8 keys at (q % 4) * 8)
+  //      piece q of V^T is (d = q / (TK/8), the 8 keys at (q % (TK/8)) * 8)
   bf16x8 kreg[PT], vreg[PT];
   auto load_tile = [&](int k0) {
 #pragma unroll
@@ -424,8 +423,8 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
       const int page = table[key / ps];
       kreg[j] = *reinterpret_cast<const bf16x8*>(p.k_cache + (((size_t)page * p.hkv + kvh) * ps + key % ps) * D +
                                                  (q % (D / 8)) * 8);
-      const int d = q >> 2;
-      const int vkey = min(k0 + (q & 3) * 8, (ke - 1) & ~7);
+      const int d = q / (TK / 8);
+      const int vkey = min(k0 + (q % (TK / 8)) * 8, (ke - 1) & ~7);
       const int vpage = table[vkey / ps];
       vreg[j] = *reinterpret_cast<const bf16x8*>(p.v_cache + (((size_t)vpage * p.hkv + kvh) * D + d) * (size_t)ps +
                                                  vkey % ps);
@@ -436,29 +435,31 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
     for (int j = 0; j < PT; ++j) {
       const int q = tid + 256 * j;
       *reinterpret_cast<bf16x8*>(ks + (q / (D / 8)) * KSTR + (q % (D / 8)) * 8) = kreg[j];
-      // a row of V^T is 8-byte aligned only (stride 72 bytes)
+      // a row of V^T is 8-byte aligned only
       const bf16x4 lo = {vreg[j][0], vreg[j][1], vreg[j][2], vreg[j][3]};
       const bf16x4 hi = {vreg[j][4], vreg[j][5], vreg[j][6], vreg[j][7]};
-      bf16_t* dst = vs + (q >> 2) * VSTR + (q & 3) * 8;
+      bf16_t* dst = vs + (q / (TK / 8)) * VSTR + (q % (TK / 8)) * 8;
       *reinterpret_cast<bf16x4*>(dst) = lo;
       *reinterpret_cast<bf16x4*>(dst + 4) = hi;
     }
   };
 
   if (kb < ke) load_tile(kb);
-  for (int k0 = kb; k0 < ke; k0 += kTileKeys) {
+  for (int k0 = kb; k0 < ke; k0 += TK) {
     __syncthreads();   // the previous tile has been read by every wave
     store_tile();
     __syncthreads();
-    if (k0 + kTileKeys < ke) load_tile(k0 + kTileKeys);
+    if (k0 + TK < ke) load_tile(k0 + TK);
     if (nrows == 0 || k0 >= my_ke) continue;   // the whole wave: nothing of this tile is visible to it
 
-    // ---- S^T for the two blocks of 16 keys
-    f32x4 s[RT][2];
+    // ---- S^T for the blocks of 16 keys
+    f32x4 s[RT][KB];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+      for (int b = 0; b < KB; ++b) s[rt][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int b = 0; b < KB; ++b)
 #pragma unroll
       for (int j = 0; j < KCH; ++j) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks + (16 * b + r16) * KSTR + 32 * j + 8 * g);
@@ -468,16 +469,17 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
       }
 
     // ---- softmax update; lane holds keys k0 + 16 b + 4 g + i of row r16
-    bf16x8 pb[RT];
+    bf16x8 pb[RT][KB / 2];
     float alpha[RT];
+    bool rescale = false;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      float sc[8];
+      float sc[4 * KB];
       float mx = -INFINITY;
       const int hi = min(row_pos[rt], ke - 1);
       const int lo = p.window > 0 ? row_pos[rt] - p.window + 1 : 0;
 #pragma unroll
-      for (int b = 0; b < 2; ++b)
+      for (int b = 0; b < KB; ++b)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = k0 + 16 * b + 4 * g + i;
@@ -490,31 +492,41 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
       const float new_max = fmaxf(run_max[rt], mx);
       const float base = new_max == -INFINITY ? 0.f : new_max;
       alpha[rt] = exp2f(run_max[rt] - base);
+      rescale = rescale || alpha[rt] != 1.f;
       float psum = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
+      for (int e = 0; e < 4 * KB; ++e) {
         const float pv = exp2f(sc[e] - base);
         psum += pv;
-        pb[rt][e] = static_cast<bf16_t>(pv);
+        pb[rt][e / 8][e % 8] = static_cast<bf16_t>(pv);
       }
       run_sum[rt] = run_sum[rt] * alpha[rt] + psum;
       run_max[rt] = new_max;
     }
-
-    // ---- O^T += V^T P^T
+    // the running maxima of most tiles after the first few do not move: skip the rescaling then
+    if (__any(rescale)) {
 #pragma unroll
-    for (int t = 0; t < DT; ++t) {
-      const bf16_t* vrow = vs + (16 * t + r16) * VSTR + 4 * g;
-      const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vrow);
-      const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vrow + 16);
-      const bf16x8 a = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        f32x4 c = acc[rt][t];
-        c[0] *= alpha[rt]; c[1] *= alpha[rt]; c[2] *= alpha[rt]; c[3] *= alpha[rt];
-        acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[rt], c, 0, 0, 0);
-      }
+        for (int t = 0; t < DT; ++t) {
+          acc[rt][t][0] *= alpha[rt]; acc[rt][t][1] *= alpha[rt];
+          acc[rt][t][2] *= alpha[rt]; acc[rt][t][3] *= alpha[rt];
+        }
     }
+
+    // ---- O^T += V^T P^T, 32 keys a step
+#pragma unroll
+    for (int h = 0; h < KB / 2; ++h)
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        const bf16_t* vrow = vs + (16 * t + r16) * VSTR + 32 * h + 4 * g;
+        const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vrow);
+        const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vrow + 16);
+        const bf16x8 a = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[rt][h], acc[rt][t], 0, 0, 0);
+      }
   }
 
   // ---- write: lane holds O[row r16][d = 16 t + 4 g + i]
@@ -551,9 +563,10 @@ static int launch_prefill_tiled(const AttnParams& p, int num_tiles, int rows_per
   const int gh = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
   if (rows_per_tile != 32 * (4 / gh)) return ATOM_BAD_SHAPE;
   dim3 grid(num_tiles, p.hq / gh), block(256);
-  if (gh == 4) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 4>), grid, block, 0, stream, p);
-  else if (gh == 2) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 2>), grid, block, 0, stream, p);
-  else hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 1>), grid, block, 0, stream, p);
+  constexpr int TK = 32;   // 64 needs so many registers that one block a CU is left, which is slower
+  if (gh == 4) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 4, TK>), grid, block, 0, stream, p);
+  else if (gh == 2) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 2, TK>), grid, block, 0, stream, p);
+  else hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 1, TK>), grid, block, 0, stream, p);
   return launch_status();
 }
 

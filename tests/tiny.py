@@ -27,7 +27,7 @@ TINY_C = dict(
     layer_types=["full_attention", "sliding_attention", "sliding_attention", "full_attention"],
     hidden_act="silu", torch_dtype="bfloat16")
 
-# the weights' spread per configuration (BASELINE: A 0.02 / 0.1, B 0.05 / 0.2)
+# the weights' spread per configuration: (linear and embedding std, norm-weight std)
 SPREAD = {"A": (0.02, 0.1), "B": (0.05, 0.2), "C": (0.04, 0.15)}
 CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 SEEDS = {"A": 0, "B": 1, "C": 5}
