@@ -138,12 +138,58 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   if (tid == 0) out[r] = best.i;
 }
 
+// Greedy rows of a large vocabulary in two steps, so that a few rows still use the whole chip: every
+// block finds the maximum of one chunk of one row (lowest index on ties), then one wave per row picks
+// among the chunks' maxima, lowest chunk first.
+constexpr int kArgmaxChunks = 64;
+
+__global__ void __launch_bounds__(256)
+argmax_chunks_kernel(const float* __restrict__ logits, float* __restrict__ ws_vals, int* __restrict__ ws_idx,
+                     int vocab) {
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  const int r = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const int per = (vocab + kArgmaxChunks - 1) / kArgmaxChunks;
+  const int lo = chunk * per, hi = min(vocab, lo + per);
+  const float* row = logits + (size_t)r * vocab;
+  MaxIdx m{-INFINITY, 0x7fffffff};
+  for (int v = lo + threadIdx.x; v < hi; v += blockDim.x) m = better(m, MaxIdx{row[v], v});
+  m = block_argmax(m, sv, si);
+  if (threadIdx.x == 0) {
+    ws_vals[r * kArgmaxChunks + chunk] = m.v;
+    ws_idx[r * kArgmaxChunks + chunk] = m.i;
+  }
+}
+
+__global__ void __launch_bounds__(kWave)
+argmax_pick_kernel(const float* __restrict__ ws_vals, const int* __restrict__ ws_idx, int* __restrict__ out) {
+  const int r = blockIdx.x;
+  MaxIdx m{ws_vals[r * kArgmaxChunks + threadIdx.x], ws_idx[r * kArgmaxChunks + threadIdx.x]};
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    MaxIdx o;
+    o.v = __shfl_xor(m.v, off, kWave);
+    o.i = __shfl_xor(m.i, off, kWave);
+    m = better(m, o);
+  }
+  if (threadIdx.x == 0) out[r] = m.i;
+}
+
+// `ws_vals` / `ws_idx` (rows * 64 elements each, or null) let all-greedy calls take the two-step path.
 ATOM_EXPORT int atom_sample(const float* logits, const float* temperatures, const int* top_ks, const float* top_ps,
                             const float* noise, long noise_stride, const unsigned long long* seeds,
                             const unsigned long long* counters, int* out, int rows, int vocab, float eps,
-                            hipStream_t stream) {
+                            float* ws_vals, int* ws_idx, hipStream_t stream) {
   if (rows < 0 || vocab <= 0) return ATOM_BAD_SHAPE;
   if (rows == 0) return ATOM_OK;
+  static_assert(kArgmaxChunks == kWave, "the pick kernel holds one chunk per lane");
+  if (!temperatures && ws_vals && ws_idx && vocab >= 16384 && rows <= 65535) {
+    hipLaunchKernelGGL(argmax_chunks_kernel, dim3(kArgmaxChunks, rows), dim3(256), 0, stream, logits, ws_vals, ws_idx,
+                       vocab);
+    hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(kWave), 0, stream, ws_vals, ws_idx, out);
+    return launch_status();
+  }
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kSampleThreads), 0, stream, logits, temperatures, top_ks,
                      top_ps, noise, noise_stride, seeds, counters, out, vocab, eps);
   return launch_status();

@@ -328,9 +328,11 @@ def test_window_edge():
 # ------------------------------------------------------------------ sampling
 
 
-def test_sample_greedy_and_ties():
-    logits = rnd((9, 517), torch.float32, 30)
-    logits[3, 100] = logits[3, 400] = 50.0   # a tie: the lower index wins
+@pytest.mark.parametrize("vocab", [517, 151936, 20001])   # large vocabularies take the two-step argmax
+def test_sample_greedy_and_ties(vocab):
+    logits = rnd((9, vocab), torch.float32, 30)
+    logits[3, 100] = logits[3, vocab - 117] = 50.0   # a tie, in different chunks: the lower index wins
+    logits[5, vocab - 1] = 60.0
     out = torch.empty(9, dtype=torch.int32, device=DEV)
     gpu_ops().sample(logits.to(DEV), None, out)
     want = logits.argmax(dim=-1)
