@@ -350,6 +350,35 @@ __global__ void qk_norm_rope_kv_write_kernel(
   const bool is_k = !is_q && head < hq + hkv;
   const int kv_head = is_q ? 0 : (is_k ? head - hq : head - hq - hkv);
 
+  if (!is_q && !is_k && write_kv && !xsum.partial && page_size % 8 == 0) {
+    // value heads of 8 consecutive tokens whose slots are 8 consecutive, aligned places of one page
+    // (the usual case in a prompt portion): the first token's wave writes all 8, 8 keys at a time per
+    // d, instead of every token scattering single elements over the transposed page
+    const int t0 = t & ~7;
+    bool together = t0 + 8 <= (int)gridDim.x;
+    int s0 = -1;
+    if (together) {
+      s0 = slots[t0];
+      together = s0 >= 0 && s0 % 8 == 0;
+      for (int j = 1; j < 8 && together; ++j) together = slots[t0 + j] == s0 + j;
+    }
+    if (together) {
+      if (t != t0) return;
+      const int page0 = s0 / page_size, off0 = s0 - page0 * page_size;
+      T* base = v_cache + ((size_t)page0 * hkv + kv_head) * (size_t)d * page_size + off0;
+      const T* rows = qkv + (size_t)t0 * row_width + (size_t)head * d;
+      for (int i = lane; i < d; i += kWave) {
+        float vals[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) vals[j] = to_f32(rows[(size_t)j * row_width + i]);
+        Vec8<T> out8;
+        out8.set(vals);
+        *reinterpret_cast<Vec8<T>*>(base + (size_t)i * page_size) = out8;
+      }
+      return;
+    }
+  }
+
   int slot = -1;
   if (!is_q) {
     if (!write_kv) return;

@@ -157,6 +157,33 @@ def test_qk_norm_rope_kv_write(dtype, hq, hkv, d, rot, page, norm):
     assert torch.equal(before_k, kc_gpu) and torch.equal(before_v, vc_gpu)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page", [8, 16, 32])
+def test_kv_write_of_token_runs(dtype, page):
+    """Runs of 8 tokens whose slots are 8 consecutive aligned places are written together; runs that are
+    shifted, broken by a padding row, cross a page or are cut short by the end take the single-token way."""
+    hq, hkv, d = 4, 2, 64
+    runs = [list(range(32, 40)), list(range(65, 73)), [96, 97, 98, -1, 100, 101, 102, 103],
+            list(range(156, 164)),   # crosses the page edge at 160
+            list(range(200, 208)), [16, 17, 18]]
+    slots = torch.tensor([s for run in runs for s in run], dtype=torch.int32)
+    tokens = slots.numel()
+    pages = 256 // page + 2
+    qkv = rnd((tokens, (hq + 2 * hkv) * d), dtype, 90, 2.0)
+    positions = torch.arange(tokens, dtype=torch.int32)
+    ang = torch.outer(torch.arange(64, dtype=torch.float32), 1.0 / (1e4 ** (torch.arange(0, d, 2) / d)))
+    cos, sin = ang.cos().contiguous(), ang.sin().contiguous()
+    kc, vc = rnd((pages, hkv, page, d), dtype, 91), rnd((pages, hkv, d, page), dtype, 92)
+    kc_gpu, vc_gpu = kc.to(DEV), vc.to(DEV)
+    q_gpu = torch.empty((tokens, hq, d), dtype=dtype, device=DEV)
+    gpu_ops().qk_norm_rope_kv_write(qkv.to(DEV), q_gpu, kc_gpu, vc_gpu, None, None, cos.to(DEV), sin.to(DEV),
+                                    positions.to(DEV), slots.to(DEV), hq, hkv, d, d, page, 1e-5)
+    q_want = torch.empty((tokens, hq, d), dtype=dtype)
+    PLAIN.qk_norm_rope_kv_write(qkv, q_want, kc, vc, None, None, cos, sin, positions, slots, hq, hkv, d, d, page, 1e-5)
+    close(kc_gpu, kc, dtype)
+    assert torch.equal(vc_gpu.cpu(), vc), "values are copied as they are, and only into their own slots"
+
+
 def _attention_case(dtype, hq, hkv, d, page, window, q_lens, ctx_lens, seed, scale_one=None):
     """A batch with its cache filled at random pages; returns what both implementations need."""
     g = torch.Generator().manual_seed(seed)
