@@ -1,7 +1,8 @@
 """Each part alone on the GPU against the plain implementation's function of the same
 name, in float32 and bfloat16; and a toy mixer with a state of its own, defined here,
 registered, built into a model through the registries and stepped through the engine
-without a change to the framework's files."""
+without a change to the framework's files; likewise a feed-forward with routing, a position
+encoding with parameters and a mixer that keeps no cache."""
 
 from dataclasses import dataclass
 from typing import ClassVar
@@ -17,8 +18,9 @@ from atom_amd.engine.context import KVBinding, StepContext
 from atom_amd.engine.core import StepEntry, build_core, load_model
 from atom_amd.kernels.hip import AttentionMeta
 from atom_amd.models.model import ModelSpec
-from atom_amd.parts import (FEED_FORWARDS, MIXERS, NORMS, GatedMLP, GroupedQueryAttention, LMHead, Mixer, ParamSpec,
-                            PartChoice, PreNormBlock, RMSNorm, RotaryEncoding, StateNeed, TokenEmbedding)
+from atom_amd.parts import (FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, FeedForward, GatedMLP,
+                            GroupedQueryAttention, LMHead, Mixer, ParamSpec, PartChoice, PositionEncoding, PreNormBlock,
+                            RMSNorm, RotaryEncoding, StateNeed, TokenEmbedding)
 from atom_amd.weights import write_random_model
 
 pytestmark = pytest.mark.gpu
@@ -340,3 +342,172 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype, tmp_path):
     finally:
         MIXERS.unregister("running_mean")
         unregister_architecture("ToyForCausalLM")
+
+
+# ------------------------------------------------------------------ toy parts of the other kinds: a feed-forward
+# with routing, a position encoding with parameters of its own, a mixer that keeps no cache
+
+
+class LearnedPositions(PositionEncoding):
+    """One learned vector per position, added to the mixer's input."""
+
+    def __init__(self, size: int, max_positions: int, prefix: str = ""):
+        super().__init__(prefix)
+        self.size, self.max_positions = size, max_positions
+
+    def param_specs(self):
+        return {"table": ParamSpec.single("positions.weight", (self.max_positions, self.size))}
+
+
+class ShiftMixer(Mixer):
+    """y_t = W (x_t + P[position of t]): no memory of other tokens, hence no cache; the position encoding is
+    a child part chosen by name, with its own checkpoint tensor."""
+
+    def __init__(self, hidden_size: int, position_encoding: PartChoice, prefix: str = ""):
+        super().__init__(prefix)
+        self.hidden_size = hidden_size
+        self.pos = position_encoding.build(POSITION_ENCODINGS, size=hidden_size, prefix=prefix)
+
+    def children(self):
+        return [self.pos]
+
+    def param_specs(self):
+        return {"mix.weight": ParamSpec.single("mix.weight", (self.hidden_size, self.hidden_size))}
+
+    def forward(self, ctx, x, cache):
+        assert cache is None
+        shifted = (x.float() + self.pos.params["table"][ctx.positions.long()].float()).to(x.dtype)
+        return ctx.ops.linear(shifted, self.params["mix.weight"])
+
+
+class RoutedFeedForward(FeedForward):
+    """Top-1 routing over small SiLU-gated experts: router logits in float32, the chosen expert's output
+    scaled by its softmax weight."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, prefix: str = ""):
+        super().__init__(prefix)
+        self.h, self.i, self.e = hidden_size, intermediate_size, num_experts
+
+    def param_specs(self):
+        specs = {"router.weight": ParamSpec.single("router.weight", (self.e, self.h))}
+        for k in range(self.e):
+            specs[f"experts.{k}.gate_up.weight"] = ParamSpec.stacked(
+                [(f"experts.{k}.gate_proj.weight", self.i), (f"experts.{k}.up_proj.weight", self.i)], (self.h,))
+            specs[f"experts.{k}.down.weight"] = ParamSpec.single(f"experts.{k}.down_proj.weight", (self.h, self.i))
+        return specs
+
+    def forward(self, ctx, x):
+        ops = ctx.ops
+        logits = ops.linear(x, self.params["router.weight"], None, out_dtype=torch.float32)
+        weight, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+        out = torch.zeros_like(x)
+        for k in range(self.e):
+            rows = (choice == k).nonzero().squeeze(1)
+            if rows.numel() == 0:
+                continue
+            act = ops.linear_silu(x[rows].contiguous(), self.params[f"experts.{k}.gate_up.weight"])
+            y = ops.materialize(ops.linear(act, self.params[f"experts.{k}.down.weight"]))
+            out[rows] = (y.float() * weight[rows, None]).to(x.dtype)
+        return out
+
+
+def routed_spec(cfg: ToyConfig) -> ModelSpec:
+    norm = PartChoice("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps})
+    dense = PartChoice("gated_mlp", {"hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size})
+    routed = PartChoice("routed_toy", {"hidden_size": cfg.hidden_size, "intermediate_size": 24, "num_experts": 3})
+    attn = PartChoice("attention", {"hidden_size": cfg.hidden_size, "num_heads": cfg.num_attention_heads,
+                                    "num_kv_heads": 2, "head_dim": cfg.head_dim,
+                                    "position_encoding": PartChoice("rotary", {"theta": 1e4, "max_positions": cfg.max_position_embeddings})})
+    shift = PartChoice("shift_toy", {"hidden_size": cfg.hidden_size, "position_encoding": PartChoice(
+        "learned_toy", {"max_positions": cfg.max_position_embeddings})})
+    blocks = [PartChoice("prenorm", {"mixer": shift if i % 2 == 0 else attn, "feed_forward": routed if i % 2 == 0 else dense,
+                                     "norm": norm}) for i in range(cfg.num_hidden_layers)]
+    return ModelSpec(cfg.vocab_size, cfg.hidden_size, blocks, norm, max_positions=cfg.max_position_embeddings)
+
+
+def plain_routed_logits(tensors, cfg: ToyConfig, ids, round_to=None):
+    x = tensors["model.embed_tokens.weight"][torch.tensor(ids)]
+    n = len(ids)
+    residual = None
+    for i in range(cfg.num_hidden_layers):
+        p = f"model.layers.{i}."
+        if residual is None:
+            residual, h = x, pm.rms_norm(x, tensors[p + "input_layernorm.weight"], cfg.rms_norm_eps)
+        else:
+            h, residual = pm.add_rms_norm(x, residual, tensors[p + "input_layernorm.weight"], cfg.rms_norm_eps)
+        if i % 2 == 0:
+            a = (h + tensors[p + "self_attn.positions.weight"][:n]) @ tensors[p + "self_attn.mix.weight"].T
+        else:
+            q = (h @ tensors[p + "self_attn.q_proj.weight"].T).view(n, cfg.num_attention_heads, cfg.head_dim)
+            k = (h @ tensors[p + "self_attn.k_proj.weight"].T).view(n, 2, cfg.head_dim)
+            v = (h @ tensors[p + "self_attn.v_proj.weight"].T).view(n, 2, cfg.head_dim)
+            cos, sin = pm.rope_angles(torch.arange(n), cfg.head_dim, 1e4)
+            o = pm.causal_attention(pm.rope_neox(q, cos, sin), pm.rope_neox(k, cos, sin), v, cfg.head_dim ** -0.5)
+            a = o.reshape(n, -1) @ tensors[p + "self_attn.o_proj.weight"].T
+        h, residual = pm.add_rms_norm(a, residual, tensors[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps)
+        if i % 2 == 0:
+            probs = torch.softmax(h @ tensors[p + "mlp.router.weight"].T, dim=-1)
+            weight, choice = probs.max(dim=-1)
+            x = torch.zeros_like(h)
+            for t in range(n):
+                e = int(choice[t])
+                pre = f"{p}mlp.experts.{e}."
+                x[t] = weight[t] * pm.gated_mlp(h[t:t + 1], tensors[pre + "gate_proj.weight"], tensors[pre + "up_proj.weight"],
+                                                tensors[pre + "down_proj.weight"])[0]
+        else:
+            x = pm.gated_mlp(h, tensors[p + "mlp.gate_proj.weight"], tensors[p + "mlp.up_proj.weight"],
+                             tensors[p + "mlp.down_proj.weight"])
+    h, _ = pm.add_rms_norm(x, residual, tensors["model.norm.weight"], cfg.rms_norm_eps)
+    return h @ tensors["lm_head.weight"].T
+
+
+def test_toy_routed_feed_forward_and_learned_positions(tmp_path):
+    """float32 only: with 8-bit mantissas a router's top-1 choice can flip on near ties, which is a
+    property of routing and not of the engine."""
+    dtype = torch.float32
+    MIXERS.register("shift_toy", ShiftMixer)
+    FEED_FORWARDS.register("routed_toy", RoutedFeedForward)
+    POSITION_ENCODINGS.register("learned_toy", LearnedPositions)
+    register_architecture("RoutedToyForCausalLM", ToyConfig, routed_spec)
+    try:
+        cfg = ToyConfig.from_dict(dict(architectures=["RoutedToyForCausalLM"], vocab_size=83, hidden_size=32,
+                                       num_hidden_layers=4, max_position_embeddings=80))
+        folder = write_random_model(str(tmp_path / "routed"), cfg, seed=6, std=0.25, norm_std=0.1, dtype=torch.float32)
+        from safetensors.torch import load_file
+        tensors = {k: v.double() for k, v in load_file(folder + "/model.safetensors").items()}
+        for name in ("model.layers.0.self_attn.positions.weight", "model.layers.2.mlp.router.weight",
+                     "model.layers.0.mlp.experts.2.up_proj.weight", "model.layers.1.mlp.gate_proj.weight"):
+            assert name in tensors
+        model, _ = load_model(folder, dtype=dtype, device=DEV)
+        core = build_core(model, gpu_ops(), dtype=dtype, device=DEV, page_size=16, num_pages=10, max_num_seqs=2)
+        assert core.storage.bindings[0] is None and core.storage.bindings[1] is not None   # only attention keeps pages
+        g = torch.Generator().manual_seed(1)
+        reqs = {r: torch.randint(0, 83, (n,), generator=g).tolist() for r, n in (("a", 60), ("b", 33))}
+        got = {r: {} for r in reqs}
+        plan = [[("a", 0, 17)], [("a", 17, 18), ("b", 0, 30)], [("a", 18, 60), ("b", 30, 31)], [("b", 31, 33)]]
+        for parts in plan:
+            logits = core.step([StepEntry(r, reqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in parts])
+            at = 0
+            for r, lo, hi in parts:
+                for pos in range(lo, hi):
+                    got[r][pos] = logits[at].cpu()
+                    at += 1
+        experts_used = set()
+        for r, ids in reqs.items():
+            want = plain_routed_logits(tensors, cfg, ids)
+            scale = float(want.abs().max())
+            for pos in range(len(ids)):
+                diff = float((got[r][pos].double() - want[pos]).abs().max())
+                assert diff <= 5e-5 * scale, f"request {r} position {pos}: {diff:.3e}"
+        # the routing did route: more than one expert was chosen in the first layer
+        h = pm.rms_norm(tensors["model.embed_tokens.weight"][torch.tensor(reqs["a"])], tensors["model.layers.0.input_layernorm.weight"], 1e-5)
+        a = (h + tensors["model.layers.0.self_attn.positions.weight"][:60]) @ tensors["model.layers.0.self_attn.mix.weight"].T
+        h2, _ = pm.add_rms_norm(a, tensors["model.embed_tokens.weight"][torch.tensor(reqs["a"])],
+                                tensors["model.layers.0.post_attention_layernorm.weight"], 1e-5)
+        experts_used = set((h2 @ tensors["model.layers.0.mlp.router.weight"].T).argmax(-1).tolist())
+        assert len(experts_used) >= 2
+    finally:
+        MIXERS.unregister("shift_toy")
+        FEED_FORWARDS.unregister("routed_toy")
+        POSITION_ENCODINGS.unregister("learned_toy")
+        unregister_architecture("RoutedToyForCausalLM")
