@@ -11,6 +11,15 @@ one slot from its first step to its end, whether the model has such state or not
 What is given back when: all pages and the slot when a request ends or is preempted
 (``close``); a window group's pages as the window passes them (``commit``).
 
+Prefix cache (optional, groups that keep every key only): a full page whose tokens have been
+run gets a chained content hash (hash of the previous page's hash and its own tokens,
+atom/model_engine/block_manager.py:181-187).  A new request takes the longest run of pages whose
+hashes match its prompt instead of computing them again, always leaving at least its last token to
+be run (block_manager.py:374-379,397).  A hash is published only after the step that filled the page
+(:558-626).  Pages are counted by reference; a page with a hash that nobody holds stays findable
+until the pool needs it: pages that never had a hash are handed out first, then the least recently
+released hashed one, which is then forgotten (atom/model_engine/block_pool.py:153-200).
+
 Free pages are handed out lowest id first (atom/model_engine/block_pool.py:153-173 hands
 out never-used blocks lowest id first), which makes reuse deterministic.  The block math
 follows atom/model_engine/block_manager.py:1109-1133 (``can_append``/``may_append``) and
@@ -20,7 +29,8 @@ follows atom/model_engine/block_manager.py:1109-1133 (``can_append``/``may_appen
 from __future__ import annotations
 
 import heapq
-from dataclasses import dataclass
+from collections import OrderedDict
+from dataclasses import dataclass, field
 
 import numpy as np
 
@@ -41,34 +51,89 @@ class GroupSpec:
 
 
 class PagePool:
-    """Free pages of one group, lowest id first."""
+    """Pages of one group, counted by reference.  Free pages without a content hash are handed out
+    lowest id first; when none is left, the hashed page released longest ago, whose hash is forgotten."""
 
     def __init__(self, num_pages: int):
         self.num_pages = num_pages
-        self._free = list(range(num_pages))
+        self._free = list(range(num_pages))      # no hash, nobody holds them
         heapq.heapify(self._free)
-        self._held = [False] * num_pages
+        self._refs = [0] * num_pages
+        self._hash: list[int | None] = [None] * num_pages
+        self._tokens: list[tuple | None] = [None] * num_pages
+        self._by_hash: dict[int, int] = {}
+        self._cached: "OrderedDict[int, None]" = OrderedDict()   # hashed, nobody holds them; oldest first
+        self.hits = 0
+        self.evictions = 0
 
     @property
     def num_free(self) -> int:
-        return len(self._free)
+        return len(self._free) + len(self._cached)
 
     def take(self) -> int:
-        if not self._free:
+        if self._free:
+            page = heapq.heappop(self._free)
+        elif self._cached:
+            page, _ = self._cached.popitem(last=False)
+            self._forget(page)
+            self.evictions += 1
+        else:
             raise OutOfPages("no free page")
-        page = heapq.heappop(self._free)
-        assert not self._held[page], f"page {page} was free and held at once"
-        self._held[page] = True
+        assert self._refs[page] == 0, f"page {page} was free and held at once"
+        self._refs[page] = 1
         return page
 
     def give(self, page: int) -> None:
-        if not (0 <= page < self.num_pages) or not self._held[page]:
+        if not (0 <= page < self.num_pages) or self._refs[page] <= 0:
             raise AssertionError(f"page {page} is given back but is not held")
-        self._held[page] = False
-        heapq.heappush(self._free, page)
+        self._refs[page] -= 1
+        if self._refs[page] == 0:
+            if self._hash[page] is not None:
+                self._cached[page] = None
+            else:
+                heapq.heappush(self._free, page)
 
     def is_held(self, page: int) -> bool:
-        return self._held[page]
+        return self._refs[page] > 0
+
+    def refs(self, page: int) -> int:
+        return self._refs[page]
+
+    # ---- content hashes
+
+    def _forget(self, page: int) -> None:
+        h = self._hash[page]
+        if h is not None and self._by_hash.get(h) == page:
+            del self._by_hash[h]
+        self._hash[page] = None
+        self._tokens[page] = None
+
+    def publish(self, page: int, content_hash: int, tokens: tuple) -> None:
+        """The held page now holds exactly ``tokens`` after the prefix ``content_hash`` chains from.  If
+        another page already answers to the hash this one stays anonymous."""
+        assert self._refs[page] > 0
+        if self._hash[page] is not None or content_hash in self._by_hash:
+            return
+        self._hash[page] = content_hash
+        self._tokens[page] = tokens
+        self._by_hash[content_hash] = page
+
+    def find(self, content_hash: int, tokens: tuple) -> int | None:
+        """The page that holds this content, or None."""
+        page = self._by_hash.get(content_hash)
+        if page is None or self._tokens[page] != tokens:
+            return None
+        return page
+
+    def share(self, page: int) -> None:
+        """One more holder of a page found by its hash."""
+        if self._refs[page] == 0:
+            del self._cached[page]
+        self._refs[page] += 1
+        self.hits += 1
+
+    def hash_of(self, page: int) -> int | None:
+        return self._hash[page]
 
 
 class StateSlots:
@@ -104,12 +169,19 @@ class _Request:
     slot: int
     fresh: bool = True        # no step has run for it yet
     serial: int = 0           # unique per ``open``: a request id that is opened again gets a new one
+    tokens: list[int] = field(default_factory=list)   # prefix cache: the tokens that are in the cache
+    hashes: list[int] = field(default_factory=list)   # prefix cache: chained hash of every full page so far
 
 
 class CacheManager:
-    def __init__(self, groups: list[GroupSpec], num_state_slots: int):
+    def __init__(self, groups: list[GroupSpec], num_state_slots: int, prefix_caching: bool = False):
         if not groups:
             groups = []
+        if prefix_caching and any(g.window is not None for g in groups):
+            raise ValueError("the prefix cache needs groups that keep every key")
+        if prefix_caching and len({g.page_size for g in groups}) > 1:
+            raise ValueError("the prefix cache needs one page size")
+        self.prefix_caching = bool(prefix_caching and groups)
         for g in groups:
             if g.page_size <= 0 or g.num_pages < 0:
                 raise ValueError(f"bad group {g}")
@@ -231,11 +303,69 @@ class CacheManager:
                         raise AssertionError(f"request {req_id!r}: page {idx} was given back and is needed again")
                     table[idx] = self.pools[gi].take()
 
-    def commit(self, req_id, cached_after: int) -> None:
-        """After a step: ``cached_after`` tokens are in the cache.  Pages of window groups that
-        no later query can see are given back."""
+    # ------------------------------------------------------------------ prefix cache
+
+    @staticmethod
+    def _chain(previous: int, tokens: tuple) -> int:
+        import xxhash
+
+        h = xxhash.xxh64()
+        h.update(previous.to_bytes(8, "little"))
+        h.update(np.asarray(tokens, dtype=np.int32).tobytes())
+        return h.intdigest()
+
+    def match_prefix(self, req_id, token_ids) -> int:
+        """For a request that holds no page yet: takes the longest run of cached pages that hold the
+        beginning of ``token_ids`` (in every group) and returns how many tokens they cover.  At least the
+        last token is left to be run."""
+        if not self.prefix_caching:
+            return 0
+        req = self._requests[req_id]
+        if any(req.tables) or req.tokens:
+            raise AssertionError(f"request {req_id!r} already holds pages")
+        page_size = self.groups[0].page_size
+        limit = (len(token_ids) - 1) // page_size
+        previous, found_pages = 0, []
+        for idx in range(limit):
+            tokens = tuple(token_ids[idx * page_size:(idx + 1) * page_size])
+            content_hash = self._chain(previous, tokens)
+            found = [pool.find(content_hash, tokens) for pool in self.pools]
+            if any(page is None for page in found):
+                break
+            found_pages.append((content_hash, found))
+            previous = content_hash
+        for content_hash, found in found_pages:
+            for gi, page in enumerate(found):
+                self.pools[gi].share(page)
+                req.tables[gi].append(page)
+            req.hashes.append(content_hash)
+        covered = len(found_pages) * page_size
+        req.tokens = [int(t) for t in token_ids[:covered]]
+        return covered
+
+    def _publish(self, req: _Request, cached_after: int) -> None:
+        page_size = self.groups[0].page_size
+        while len(req.hashes) < cached_after // page_size:
+            idx = len(req.hashes)
+            tokens = tuple(req.tokens[idx * page_size:(idx + 1) * page_size])
+            content_hash = self._chain(req.hashes[-1] if req.hashes else 0, tokens)
+            req.hashes.append(content_hash)
+            for gi, pool in enumerate(self.pools):
+                pool.publish(req.tables[gi][idx], content_hash, tokens)
+
+    def commit(self, req_id, cached_after: int, tokens=None) -> None:
+        """After a step: ``cached_after`` tokens are in the cache (``tokens``: the ones this step ran,
+        which the prefix cache needs to name the pages they filled).  Pages of window groups that no
+        later query can see are given back."""
         req = self._requests[req_id]
         req.fresh = False
+        if self.prefix_caching:
+            if tokens is None:
+                raise ValueError("the prefix cache needs the tokens of every step")
+            req.tokens.extend(int(t) for t in tokens)
+            if len(req.tokens) != cached_after:
+                raise AssertionError(f"request {req_id!r}: {len(req.tokens)} tokens noted, {cached_after} in the cache")
+            self._publish(req, cached_after)
         for gi, g in enumerate(self.groups):
             if g.window is None:
                 continue
@@ -265,18 +395,25 @@ class CacheManager:
     # ------------------------------------------------------------------ checks
 
     def check(self) -> None:
-        """No page lost, none held twice, none both free and held; same for slots."""
+        """No page lost; every page held exactly as often as it is counted (more than once only through
+        the prefix cache); none both free and held; same for slots."""
         for gi, (g, pool) in enumerate(zip(self.groups, self.pools)):
-            held = []
+            held: dict[int, int] = {}
             for req in self._requests.values():
-                held.extend(p for p in req.tables[gi] if p >= 0)
-            assert len(held) == len(set(held)), f"group {gi}: a page is held twice"
-            free = list(pool._free)
+                for p in req.tables[gi]:
+                    if p >= 0:
+                        held[p] = held.get(p, 0) + 1
+            if not self.prefix_caching:
+                assert all(n == 1 for n in held.values()), f"group {gi}: a page is held twice"
+            for p, n in held.items():
+                assert pool.refs(p) == n, f"group {gi}: page {p} is held {n} times but counted {pool.refs(p)}"
+            free = list(pool._free) + list(pool._cached)
             assert len(free) == len(set(free)), f"group {gi}: a page is free twice"
             assert not (set(free) & set(held)), f"group {gi}: a page is free and held"
             assert len(free) + len(held) == g.num_pages, f"group {gi}: {g.num_pages - len(free) - len(held)} page(s) lost"
-            for p in held:
-                assert pool.is_held(p)
+            assert all(pool.refs(p) == 0 for p in free)
+            for h, p in pool._by_hash.items():
+                assert pool.hash_of(p) == h
         slots = [r.slot for r in self._requests.values()]
         assert len(slots) == len(set(slots)), "a state slot is held twice"
         assert len(slots) + self.slots.num_free == self.slots.num_slots, "a state slot is lost"

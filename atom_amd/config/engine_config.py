@@ -21,7 +21,7 @@ class Config:
     kv_cache_block_size: int = 16
     num_kvcache_blocks: int = -1
     kv_cache_dtype: str = "bf16"
-    enable_prefix_caching: bool = False
+    enable_prefix_caching: bool = True
     enable_chunked_prefill: bool = True
     long_prefill_token_threshold: int = 0
     scheduler_delay_factor: float = 0.0

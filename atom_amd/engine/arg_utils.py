@@ -35,7 +35,7 @@ def parse_size_list(text: str) -> list[int]:
 class EngineArgs:
     model: str = "Qwen/Qwen3-0.6B"
     enforce_eager: bool = False
-    enable_prefix_caching: bool = False
+    enable_prefix_caching: bool = True
     kv_cache_dtype: str = "bf16"
     block_size: int = 16
     max_model_len: int | None = None
@@ -57,8 +57,8 @@ class EngineArgs:
     def add_cli_args(parser: argparse.ArgumentParser) -> argparse.ArgumentParser:
         parser.add_argument("--model", type=str, default="Qwen/Qwen3-0.6B", help="Model folder (config.json + safetensors).")
         parser.add_argument("--enforce-eager", action="store_true", help="Never replay captured HIP graphs.")
-        parser.add_argument("--enable-prefix-caching", action=argparse.BooleanOptionalAction, default=False,
-                            help="Accepted for compatibility; prefix caching is not built.")
+        parser.add_argument("--enable-prefix-caching", action=argparse.BooleanOptionalAction, default=True,
+                            help="Reuse cache pages that already hold the beginning of a new prompt.")
         parser.add_argument("--kv-cache-dtype", choices=["bf16"], default="bf16", help="KV cache type (the model's own).")
         parser.add_argument("--block-size", type=int, default=16, help="Tokens per KV cache block.")
         parser.add_argument("--max-model-len", type=int, default=None, help="Longest sequence (prompt + output).")

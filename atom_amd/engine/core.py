@@ -38,13 +38,19 @@ class StepEntry:
 
 class EngineCore:
     def __init__(self, model, ops, plan: CachePlan, max_num_seqs: int, device, dtype: torch.dtype,
-                 graph_sizes: list[int] | None = None, max_model_len: int = 0):
+                 graph_sizes: list[int] | None = None, max_model_len: int = 0, prefix_caching: bool = False):
         self.model = model
         self.ops = ops
         self.device = torch.device(device)
         self.dtype = dtype
         self.plan = plan
-        self.manager = CacheManager(plan.groups, max_num_seqs)
+        # the prefix cache needs every mixer's memory to be pages that keep all keys
+        from ..parts.base import KVCacheNeed
+
+        needs = [model.blocks[run.layer].mixer.cache_need() for run in model.order]
+        self.prefix_caching = bool(prefix_caching and plan.groups and all(
+            isinstance(n, KVCacheNeed) and n.window is None for n in needs if n is not None))
+        self.manager = CacheManager(plan.groups, max_num_seqs, prefix_caching=self.prefix_caching)
         self.storage = CacheStorage(model, plan, max_num_seqs, self.device, dtype)
         self.lengths: dict[object, int] = {}   # tokens of each live request that are in the cache
         self.max_positions = model.spec.max_positions
@@ -74,6 +80,15 @@ class EngineCore:
         self.manager.open(req_id)
         self.lengths[req_id] = 0
         self._fresh_slots.append(self.manager.state_slot(req_id))
+
+    def match_prefix(self, req_id, token_ids) -> int:
+        """For a request just opened: takes cached pages that already hold the beginning of ``token_ids``
+        and returns how many tokens need not be run (0 without a prefix cache)."""
+        if not self.prefix_caching or self.lengths.get(req_id, 0) != 0:
+            return 0
+        covered = self.manager.match_prefix(req_id, token_ids)
+        self.lengths[req_id] = covered
+        return covered
 
     def close(self, req_id) -> None:
         """Ends a request: its pages and state slot go back."""
@@ -142,7 +157,7 @@ class EngineCore:
 
         for e in entries:
             self.lengths[e.req_id] += len(e.tokens)
-            self.manager.commit(e.req_id, self.lengths[e.req_id])
+            self.manager.commit(e.req_id, self.lengths[e.req_id], e.tokens if self.prefix_caching else None)
         self.steps_run += 1
         return logits
 
@@ -252,11 +267,12 @@ def load_model(model_dir: str | None, *, dtype: torch.dtype, device, model_confi
 
 def build_core(model, ops, *, dtype: torch.dtype, device, page_size: int = 16, num_pages: int | None = None,
                budget_bytes: int | None = None, max_num_seqs: int = 4, max_model_len: int = 0,
-               max_num_batched_tokens: int = 0, graph_sizes: list[int] | None = None) -> EngineCore:
+               max_num_batched_tokens: int = 0, graph_sizes: list[int] | None = None,
+               prefix_caching: bool = False) -> EngineCore:
     from ..cache.storage import plan_cache
 
     plan = plan_cache(model, page_size, dtype, num_pages=num_pages, budget_bytes=budget_bytes,
                       max_num_seqs=max_num_seqs, max_model_len=max_model_len,
                       max_num_batched_tokens=max_num_batched_tokens)
     return EngineCore(model, ops, plan, max_num_seqs, device, dtype, graph_sizes=graph_sizes,
-                      max_model_len=max_model_len)
+                      max_model_len=max_model_len, prefix_caching=prefix_caching)

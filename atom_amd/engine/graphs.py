@@ -15,6 +15,8 @@ Buckets are captured on first use.  Every captured graph shares one memory pool.
 
 from __future__ import annotations
 
+import gc
+
 import numpy as np
 import torch
 
@@ -167,8 +169,18 @@ class DecodeGraphs:
         if self.pool is None:
             self.pool = torch.cuda.graph_pool_handle()
         cap.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(cap.graph, pool=self.pool, stream=stream):
-            cap.logits = core.model.forward(ctx, tokens, core.storage.bindings, want)
+        # No garbage collection while the stream is capturing: a collected tensor, event or older graph
+        # frees device objects, which is not allowed during capture and aborts the process (the reference
+        # pauses it for the same reason, atom/model_engine/model_runner.py:4046-4055).
+        gc.collect()
+        gc_was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(cap.graph, pool=self.pool, stream=stream):
+                cap.logits = core.model.forward(ctx, tokens, core.storage.bindings, want)
+        finally:
+            if gc_was_enabled:
+                gc.enable()
         self.captured[size] = cap
         return cap
 

@@ -41,8 +41,6 @@ class LLMEngine:
     def __init__(self, model: str, tokenizer=None, ops=None, weight_source=None, **kwargs):
         kwargs = {k: v for k, v in kwargs.items() if k in Config.__dataclass_fields__}
         self.config = cfg = Config(model, **kwargs)
-        if cfg.enable_prefix_caching:
-            logger.warning("prefix caching is not built in this engine; running without it")
         self.tokenizer = tokenizer if tokenizer is not None else (
             _load_tokenizer(model) if isinstance(model, str) and os.path.isdir(model) else None)
         self.dtype = TORCH_DTYPES[cfg.dtype]
@@ -65,7 +63,8 @@ class LLMEngine:
             budget_bytes=self._cache_budget() if cfg.num_kvcache_blocks <= 0 else None,
             max_num_seqs=cfg.max_num_seqs, max_model_len=cfg.max_model_len,
             max_num_batched_tokens=cfg.max_num_batched_tokens,
-            graph_sizes=None if cfg.enforce_eager else cfg.cudagraph_capture_sizes)
+            graph_sizes=None if cfg.enforce_eager else cfg.cudagraph_capture_sizes,
+            prefix_caching=cfg.enable_prefix_caching)
         self.scheduler = Scheduler(cfg, self.core)
         self.sampler = Sampler(ops, cfg.device)
         self.seqs: dict[int, Sequence] = {}

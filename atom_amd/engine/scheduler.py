@@ -7,8 +7,9 @@ budget with a truncated portion floored to a multiple of ``max(block_size, 64)``
 sliver not scheduled unless the batch is empty (:1733-1753), permanent rejection of
 requests that can never run (:989-1050), preemption of the last running request when
 pages run out, the preempted request going back to the head of the waiting queue and
-later prefilling prompt plus generated tokens (:1917-1952, :1277-1283), and the finishing
-rules in their order (:2296-2329).
+later prefilling prompt plus generated tokens (:1917-1952, :1277-1283), the finishing
+rules in their order (:2296-2329), and with the prefix cache on a new request starting after the
+pages that already hold its beginning (``num_new = num_tokens - hits * block``, :1187-1347).
 
 What differs: the reference schedules prompt portions *or* decode tokens per step
 (:1370-1429); here one step holds both.  Running requests that decode are scheduled
@@ -237,19 +238,24 @@ class Scheduler:
             if len(self.running) >= self.max_num_seqs or not mgr.can_open():
                 self.waiting.appendleft(seq)
                 break
-            num_new = seq.num_tokens
+            # the request is opened first: pages that already hold the beginning of its tokens (prefix
+            # cache) are taken before the rest is counted
+            self.core.open(seq.id)
+            hit = self.core.match_prefix(seq.id, seq.token_ids)
+            num_new = seq.num_tokens - hit
             if self.enable_chunked_prefill and 0 < self.long_prefill_token_threshold < num_new:
                 num_new = self.long_prefill_token_threshold
             chunk = self._prefill_chunk_for_budget(num_new, self.max_num_batched_tokens - batched, batched)
-            if chunk is None or not mgr.can_cover(seq.id, 0, chunk, seq.num_tokens):
+            if chunk is None or not mgr.can_cover(seq.id, hit, hit + chunk, seq.num_tokens):
+                self.core.close(seq.id)
                 self.waiting.appendleft(seq)
                 break
-            self.core.open(seq.id)
-            mgr.cover(seq.id, 0, chunk, seq.num_tokens)
+            mgr.cover(seq.id, hit, hit + chunk, seq.num_tokens)
             seq.status = SequenceStatus.RUNNING
-            seq.num_cached_tokens = 0
+            seq.num_cached_tokens = hit
+            seq.num_prefix_hit_tokens = hit
             self.running.append(seq)
-            batch.items.append(ScheduledItem(seq, chunk, 0, False, chunk >= seq.num_tokens))
+            batch.items.append(ScheduledItem(seq, chunk, hit, False, hit + chunk >= seq.num_tokens))
             scheduled.add(seq.id)
             batched += chunk
 

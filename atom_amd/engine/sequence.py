@@ -37,6 +37,7 @@ class Sequence:
         self.leave_reason = ""
         self.logprobs: list[float] = []
         self.num_preemptions = 0
+        self.num_prefix_hit_tokens = 0      # tokens of the last admission that came from the prefix cache
         self.arrive_time = time.time()
         self.first_token_time = 0.0
         self.leave_time = 0.0

@@ -61,6 +61,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--points", type=str, default="1,64", help="other decode batch sizes to time")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--mixed", type=int, default=0, metavar="N",
+                    help="instead: N requests with prompts of 64..3072 tokens through the scheduler, prompt portions of "
+                         "512 tokens beside running decodes, 128 output tokens each; prints its own line")
     ap.add_argument("--enforce-eager", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -78,7 +81,8 @@ def main() -> int:
     raw["num_hidden_layers"] = layers
     cfg = model_config_from_dict(raw)
     points = sorted({int(x) for x in args.points.split(",") if x} | {args.batch})
-    max_seqs = max(points)
+    points = [p for p in points]
+    max_seqs = max(points + [args.mixed])
     max_model_len = 4096
     block = 16
     t0 = time.time()
@@ -96,6 +100,28 @@ def main() -> int:
 
     def sync():
         torch.cuda.synchronize()
+
+    if args.mixed:
+        # continuous batching under load: every step holds the running requests' decode tokens and, under a
+        # budget of 512 + N tokens, the next portion of a waiting prompt
+        llm.scheduler.max_num_batched_tokens = 512 + args.mixed
+        lens = torch.randint(64, 3073, (args.mixed,), generator=gen).tolist()
+        sp = SamplingParams(temperature=0.0, max_tokens=128, ignore_eos=True)
+        prompts = [torch.randint(0, vocab, (n,), generator=gen).tolist() for n in lens]
+        sync()
+        t = time.perf_counter()
+        outs = llm.generate(prompts, sp)
+        sync()
+        elapsed = time.perf_counter() - t
+        assert all(o["num_tokens_output"] == 128 for o in outs)
+        print(json.dumps({"workload": "mixed", "requests": args.mixed, "prompt_tokens": sum(lens),
+                          "output_tokens": 128 * args.mixed, "seconds": round(elapsed, 3),
+                          "output_tok_s": round(128 * args.mixed / elapsed, 1),
+                          "total_tok_s": round((sum(lens) + 128 * args.mixed) / elapsed, 1),
+                          "steps": llm.core.steps_run, "preemptions": llm.scheduler.total_preemptions,
+                          "mean_ttft_ms": round(1e3 * sum(o["ttft"] for o in outs) / len(outs), 1),
+                          "mean_tpot_ms": round(1e3 * sum(o["tpot"] for o in outs) / len(outs), 2)}), flush=True)
+        return 0
 
     # ---- prefill of one 2,048-token prompt
     prefill = None

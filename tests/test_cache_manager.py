@@ -206,3 +206,100 @@ def test_plan_groups_layers_by_window():
     per_req = -(-(40 + 64) // 16) + 1
     assert plan.groups[1].num_pages == 4 * per_req
     assert plan.groups[0].num_pages == ((10 << 20) - 4 * per_req * plan.bytes_per_page[1]) // plan.bytes_per_page[0]
+
+
+# ------------------------------------------------------------------ prefix cache
+
+
+def _run(m, rid, tokens, start=0):
+    """Takes pages for ``tokens`` at ``start`` and notes them as run."""
+    m.cover(rid, start, start + len(tokens))
+    m.commit(rid, start + len(tokens), tokens)
+
+
+def test_pool_prefers_pages_without_a_hash_then_the_oldest_hashed():
+    """Free order of the reference's pool (tests/test_block_pool.py:26-60): vacant pages first, lowest id first;
+    then hashed pages in the order they were released; a page that is handed out again forgets its hash."""
+    pool = PagePool(4)
+    pages = [pool.take() for _ in range(4)]
+    pool.publish(1, 111, (1,))
+    pool.publish(2, 222, (2,))
+    for p in (2, 0, 1, 3):
+        pool.give(p)
+    assert pool.num_free == 4
+    assert pool.find(222, (2,)) == 2 and pool.find(222, (9,)) is None, "a hash answers only for its own tokens"
+    assert [pool.take() for _ in range(3)] == [0, 3, 2]     # vacant 0, 3, then 2 (released before 1)
+    assert pool.find(222, (2,)) is None and pool.find(111, (1,)) == 1
+    pool.share(1)                                            # found by content: held again, no longer evictable
+    with pytest.raises(OutOfPages):
+        pool.take()
+    assert pool.refs(1) == 1 and pages == [0, 1, 2, 3]
+
+
+def test_hash_is_published_only_after_the_step_and_chains_over_the_prefix():
+    m = CacheManager([GroupSpec(4, 10)], 4, prefix_caching=True)
+    prompt = [5, 6, 7, 8, 9, 10, 11, 12, 13]
+    m.open("a")
+    m.cover("a", 0, 9)
+    m.open("b")
+    assert m.match_prefix("b", prompt) == 0, "pages are taken but nothing has been run yet"
+    m.commit("a", 9, prompt)
+    m.close("b")
+    m.open("b")
+    assert m.match_prefix("b", prompt) == 8 and m.block_table("b", 0) == m.block_table("a", 0)[:2]
+    m.open("c")
+    assert m.match_prefix("c", [0, 0, 0, 0] + prompt[4:]) == 0, "same second page, other prefix: no hit"
+    m.open("d")
+    assert m.match_prefix("d", prompt[:8]) == 4, "the last token is always left to run"
+    m.check()
+    m.close("a")
+    m.check()
+    assert m.num_free_pages() == 10 - 2, "b still holds the two shared pages"
+    for r in ("b", "c", "d"):
+        m.close(r)
+    assert m.num_free_pages() == 10
+    m.open("e")
+    assert m.match_prefix("e", prompt) == 8, "released pages stay findable until the pool needs them"
+    m.check()
+
+
+def test_prefix_cache_random_orders():
+    rng = random.Random(5)
+    m = CacheManager([GroupSpec(4, 24), GroupSpec(4, 24)], 4, prefix_caching=True)
+    stems = [[rng.randrange(50) for _ in range(12)] for _ in range(3)]
+    live = {}
+    for step in range(400):
+        if live and (len(live) == 4 or rng.random() < 0.4):
+            rid = rng.choice(list(live))
+            tokens, at = live[rid]
+            if at >= len(tokens) or rng.random() < 0.1:
+                m.close(rid)
+                del live[rid]
+            else:
+                n = min(rng.choice([1, 1, 2, 5]), len(tokens) - at)
+                if m.can_cover(rid, at, at + n):
+                    _run(m, rid, tokens[at:at + n], at)
+                    live[rid] = (tokens, at + n)
+                else:
+                    m.close(rid)
+                    del live[rid]
+        else:
+            rid = f"r{step}"
+            tokens = rng.choice(stems)[:rng.randrange(4, 13)] + [rng.randrange(50) for _ in range(rng.randrange(0, 9))]
+            m.open(rid)
+            hit = m.match_prefix(rid, tokens)
+            assert hit % 4 == 0 and hit < len(tokens)
+            for gi in range(2):
+                assert len(m.block_table(rid, gi)) == hit // 4
+            live[rid] = (tokens, hit)
+        m.check()
+    assert m.pools[0].hits > 20
+    for rid in list(live):
+        m.close(rid)
+    m.check()
+    assert m.num_free_pages(0) == 24 and m.num_free_pages(1) == 24
+
+
+def test_prefix_cache_refuses_window_groups():
+    with pytest.raises(ValueError):
+        CacheManager([GroupSpec(4, 8, window=6)], 2, prefix_caching=True)

@@ -138,3 +138,34 @@ def test_command_line():
     prompts = [[rng.randrange(256) for _ in range(n)] for n in (5, 17, 33)]
     shown = [eval(m) for m in re.findall(r"Completion: (\[.*?\])", res.stdout)]
     check_greedy("A", "fp32", prompts, [{"token_ids": ids} for ids in shown])
+
+
+@pytest.mark.parametrize("which,dtype", [("A", "fp32"), ("B", "fp32"), ("B", "bf16")])
+def test_prefix_cache_reuses_pages_and_changes_nothing(which, dtype):
+    """Requests that begin alike: with the prefix cache the later ones start after the pages that hold
+    their beginning; the tokens are those of an engine without it (and of the plain implementation)."""
+    stem = random_ids(which, 70, 3)
+    prompts = [stem, stem + random_ids(which, 9, 4), stem[:41] + random_ids(which, 20, 5), stem]
+    sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    outs = {}
+    for caching in (True, False):
+        llm = engine(which, dtype, enable_prefix_caching=caching, max_num_seqs=2)
+        assert llm.core.prefix_caching == caching
+        outs[caching] = [llm.generate([p], sp)[0] for p in prompts[:2]] + llm.generate(prompts[2:], sp)
+        llm.core.manager.check()
+        pool = llm.core.manager.pools[0]
+        assert pool.num_free == pool.num_pages
+        if caching:
+            page = PAGE[which]
+            # the 2nd finds the 1st's prompt pages, the 3rd 41 tokens' worth, the 4th all but its last page
+            assert pool.hits >= (70 // page) + (41 // page) + (69 // page)
+        else:
+            assert pool.hits == 0
+    if dtype == "fp32":
+        assert [o["token_ids"] for o in outs[True]] == [o["token_ids"] for o in outs[False]]
+    check_greedy(which, dtype, prompts, outs[True])
+
+
+def test_prefix_cache_is_off_where_a_window_gives_pages_back():
+    llm = engine("C", "fp32", enable_prefix_caching=True)
+    assert not llm.core.prefix_caching

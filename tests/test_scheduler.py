@@ -16,19 +16,22 @@ from tiny import TINY_C
 class FakeCore:
     """What the scheduler needs of the engine core: the cache manager and open/close."""
 
-    def __init__(self, groups, slots):
-        self.manager = CacheManager(groups, slots)
+    def __init__(self, groups, slots, prefix_caching=False):
+        self.manager = CacheManager(groups, slots, prefix_caching=prefix_caching)
 
     def open(self, rid):
         if rid not in self.manager:
             self.manager.open(rid)
+
+    def match_prefix(self, rid, token_ids):
+        return self.manager.match_prefix(rid, token_ids)
 
     def close(self, rid):
         if rid in self.manager:
             self.manager.close(rid)
 
 
-def make(blocks=100, block=4, window_group=None, **kw):
+def make(blocks=100, block=4, window_group=None, prefix_caching=False, **kw):
     raw = {**TINY_C, "max_position_embeddings": 4096, "eos_token_id": 2}
     kw.setdefault("max_num_seqs", 4)
     kw.setdefault("max_num_batched_tokens", 64)
@@ -37,7 +40,7 @@ def make(blocks=100, block=4, window_group=None, **kw):
     groups = [GroupSpec(block, blocks)]
     if window_group:
         groups.append(GroupSpec(block, window_group[1], window=window_group[0]))
-    core = FakeCore(groups, cfg.max_num_seqs)
+    core = FakeCore(groups, cfg.max_num_seqs, prefix_caching)
     return Scheduler(cfg, core), core
 
 
@@ -48,6 +51,9 @@ def seq(tokens, **sp):
 def run(sched, batch, token=5):
     """Pretends the step ran: every final item samples ``token``."""
     sampled = {it.seq.id: (token(it.seq) if callable(token) else token) for it in batch.items if it.is_final}
+    if sched.manager.prefix_caching:   # what the step function does after running the tokens
+        for it in batch.items:
+            sched.manager.commit(it.seq.id, it.start + it.num_tokens, it.seq.token_ids[it.start:it.start + it.num_tokens])
     return sched.postprocess(batch, sampled)
 
 
@@ -273,3 +279,48 @@ def test_aborted_waiting_request_leaves_without_running():
     sched.add(s)
     assert sched.schedule() is None
     assert sched.take_rejected() == [s] and s.leave_reason == "aborted"
+
+
+# ------------------------------------------------------------------ prefix cache
+
+
+def test_new_request_starts_after_the_pages_that_hold_its_beginning():
+    sched, core = make(blocks=20, block=4, prefix_caching=True)
+    prompt = list(range(10, 20))
+    a = seq(prompt, max_tokens=1)
+    sched.add(a)
+    batch = sched.schedule()
+    assert [(it.start, it.num_tokens) for it in batch.items] == [(0, 10)]
+    assert run(sched, batch) == [a]                      # finished; its two full pages stay findable
+    b = seq(prompt + [99, 98], max_tokens=2)
+    c = seq(prompt[:6] + [1, 2, 3], max_tokens=2)          # shares only the first page
+    sched.extend([b, c])
+    batch = sched.schedule()
+    assert [(it.seq.id, it.start, it.num_tokens) for it in batch.items] == [(b.id, 8, 4), (c.id, 4, 5)]
+    assert core.manager.block_table(b.id, 0)[0] == core.manager.block_table(c.id, 0)[0]   # one page, two holders
+    run(sched, batch)
+    core.manager.check()
+    # the same prompt again: all but the last token's page comes from the cache, never the whole prompt
+    d = seq(prompt[:8], max_tokens=1)
+    sched.add(d)
+    batch = sched.schedule()
+    item = [it for it in batch.items if it.seq is d][0]
+    assert (item.start, item.num_tokens) == (4, 4), "at least the last token is run"
+
+
+def test_preempted_request_finds_its_own_pages_again():
+    sched, core = make(blocks=6, block=4, prefix_caching=True, max_num_seqs=2)
+    a, b = seq(range(100, 108), max_tokens=20, ignore_eos=True), seq(range(200, 208), max_tokens=20, ignore_eos=True)
+    sched.extend([a, b])
+    run(sched, sched.schedule())
+    steps = 0
+    while sched.total_preemptions == 0 and steps < 20:
+        run(sched, sched.schedule())
+        steps += 1
+    assert sched.total_preemptions == 1 and b.status == SequenceStatus.WAITING
+    core.manager.check()
+    while a.status != SequenceStatus.FINISHED:
+        run(sched, sched.schedule())
+    batch = sched.schedule()
+    item = [it for it in batch.items if it.seq is b][0]
+    assert item.start >= 8, "the pages it filled before it was preempted are found by their content"
