@@ -144,7 +144,10 @@ def main() -> int:
 
     # ---- decode at each batch size
     def decode(batch: int, steps: int, warmup: int):
-        sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + 1, ignore_eos=True)
+        # prompts are admitted over several steps, so the first requests are some tokens ahead of the last
+        # when all decode: leave room, so that none finishes (and the batch does not shrink) while timed
+        admission_steps = -(-batch * args.context // 16384) + 1
+        sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + admission_steps + 2, ignore_eos=True)
         for _ in range(batch):
             llm.add_request(prompt(), sp)
         while any(s.num_completion_tokens == 0 for s in llm.seqs.values()):   # prompts, untimed
@@ -152,12 +155,14 @@ def main() -> int:
         for _ in range(warmup):
             llm.step()
         sync()
+        assert len(llm.scheduler.running) == batch and not llm.scheduler.waiting
         start_ctx = next(iter(llm.seqs.values())).num_tokens
         t = time.perf_counter()
         for _ in range(steps):
             llm.step()
         sync()
         elapsed = time.perf_counter() - t
+        assert len(llm.scheduler.running) == batch, "a request finished inside the timed steps"
         while not llm.is_finished():
             llm.step()
         llm.seqs.clear()
