@@ -10,7 +10,8 @@ padded the reference's way (model_runner.py:2577-2590): padding rows have token 
 context length 0 (attention sees no key), cache slot -1 (nothing is written) and
 request index -1.
 
-Buckets are captured on first use.  Every captured graph shares one memory pool.
+Buckets are captured on first use, or all at once with ``capture_all`` (the engine does that when it
+is built).  Every captured graph shares one memory pool.
 """
 
 from __future__ import annotations
@@ -183,6 +184,15 @@ class DecodeGraphs:
                 gc.enable()
         self.captured[size] = cap
         return cap
+
+    def capture_all(self) -> int:
+        """Captures every bucket now, largest first (atom/model_engine/model_runner.py:3973), so that no
+        step of a running engine pays for a capture.  Returns how many graphs there are."""
+        if self.usable:
+            for size in sorted(self.sizes, reverse=True):
+                if size not in self.captured:
+                    self._capture(size)
+        return len(self.captured)
 
     def run(self, entries, cached: list[int]) -> torch.Tensor:
         """Float32 logits [len(entries), vocab] of the entries' single tokens."""

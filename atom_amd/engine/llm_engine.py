@@ -65,6 +65,8 @@ class LLMEngine:
             max_num_batched_tokens=cfg.max_num_batched_tokens,
             graph_sizes=None if cfg.enforce_eager else cfg.cudagraph_capture_sizes,
             prefix_caching=cfg.enable_prefix_caching)
+        if self.core.graphs is not None:   # as the reference's engine does before it serves (engine_core.py:131-138)
+            self.core.graphs.capture_all()
         self.scheduler = Scheduler(cfg, self.core)
         self.sampler = Sampler(ops, cfg.device)
         self.seqs: dict[int, Sequence] = {}
@@ -120,7 +122,8 @@ class LLMEngine:
         if batch is None:
             return done
         start = time.time()
-        logits = self.core.step(batch.entries())
+        with torch.profiler.record_function(self._run_label(batch)):
+            logits = self.core.step(batch.entries())
         sampled = {}
         finals = [it for it in batch.items if it.is_final]
         if finals:
@@ -136,6 +139,20 @@ class LLMEngine:
                     it.seq.logprobs.append(lps[k])
         done += self.scheduler.postprocess(batch, sampled, time.time() - start)
         return done
+
+    @staticmethod
+    def _run_label(batch) -> str:
+        """The span name of a step in a profiler trace, in the reference's form
+        (atom/model_engine/run_labels.py:1-37): ``prefill[bs=2 tok=96 ctx=160]``, ``decode[bs=8 ctx=..]``."""
+        prefill = [it for it in batch.items if not it.is_decode]
+        decode = [it for it in batch.items if it.is_decode]
+        parts = []
+        if prefill:
+            parts.append(f"prefill[bs={len(prefill)} tok={sum(it.num_tokens for it in prefill)} "
+                         f"ctx={sum(it.start + it.num_tokens for it in prefill)}]")
+        if decode:
+            parts.append(f"decode[bs={len(decode)} ctx={sum(it.start + 1 for it in decode)}]")
+        return "+".join(parts)
 
     # ------------------------------------------------------------------ generate
 
