@@ -3,23 +3,21 @@
 // weight matrix is streamed from memory once and the work is bound by that stream.
 //
 // A block of four waves owns 64 rows of w (64 output columns) and a slice of K; each
-// wave owns 16 of the rows.  The weights are the A operand of v_mfma_f32_16x16x32_bf16
-// and are loaded from memory straight into the operand layout (lane (r, g) holds
-// w[row r][k + 8 g .. k + 8 g + 7], 16 bytes), a chunk of 256 k ahead of the chunk being
-// multiplied.  x is the B operand; the block's slice of it is staged in LDS and shared
-// by the four waves, so x is read from the cache hierarchy once per 64 rows of w.
-// Blocks that are neighbours in the grid read neighbouring slices of the same rows.
+// wave owns 16 of the rows and walks its part of the slice in shots of 512 k.  For a shot
+// a wave issues all its 16 loads at once, non-temporal, each covering 256 contiguous
+// bytes of four rows (whole cache lines: lanes 16 q .. 16 q + 15 read k 128 s .. 128 s + 127
+// of row 4 rg + q for load (rg, s)).  The matrix cores want the weights as the A operand of
+// v_mfma_f32_16x16x32_bf16 (lane (r, g) holds w[row r][k + 8 g .. k + 8 g + 7]), so each
+// quarter of the shot goes through a small wave-private LDS area to change layout.  x is
+// the B operand; the block's slice of it is staged in LDS and shared by the four waves, so
+// x is read from the cache hierarchy once per 64 rows of w.  Blocks that are neighbours in
+// the grid read neighbouring slices of the same rows.
 //
 // When N / 64 blocks would not fill the chip, K is cut into `splits` slices and every
 // block writes its partial tile to partial[split][m][n] (float32).  Whoever reads the
 // product next adds the slices in slice order: the norm, the rotation kernel, SiLU-mul,
 // or atom_splitk_reduce.  The sum has one fixed order, so a row's result does not
 // depend on its batch.
-//
-// A wide product (256 row tiles or more: the gate/up and head products) runs with sixteen waves a
-// block instead: four groups of four waves share the block's rows and x slice and each take a
-// quarter of its K, and their sums are added through LDS in group order.  That puts enough loads
-// in flight without cutting K between blocks, so the epilogue can be applied at once.
 //
 // Epilogues when K is not cut: plain (bias optional, bfloat16 or float32 out), or
 // SiLU-gate: w holds `inter` gate rows then `inter` up rows, a block owns 32 columns of
@@ -41,23 +39,25 @@ struct SkinnyParams {
 };
 
 struct SkinnyPlan {
-  int splits, kslice, xk, kgroups;
+  int splits, kslice, xk;
 };
 
 constexpr int kSkinnyRows = 64;    // rows of w per block
-constexpr int kSkinnyChunk = 256;  // k elements per chunk
-constexpr int kSkinnyU = kSkinnyChunk / 32;
+constexpr int kSkinnyChunk = 512;  // k elements per shot
 constexpr int kSkinnyLds = 64 * 1024;
+constexpr int kARow = 256 + 16;    // LDS bytes of one row of a quarter shot (128 k), padded by 4 banks
+constexpr int kAWave = 16 * kARow; // LDS bytes of a wave's layout-change area
 
-template <int MT, bool GATE, int KG>
-__global__ void __launch_bounds__(256 * KG) gemm_skinny_kernel(SkinnyParams p) {
-  constexpr int U = kSkinnyU;
-  constexpr int THREADS = 256 * KG;
-  extern __shared__ __attribute__((aligned(16))) char smem[];   // x slice; later the float32 tiles
+template <int MT, bool GATE>
+__global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
+  constexpr int THREADS = 256;
+  // [a wave's layout-change area] x 4, then the x slice (later the float32 tile)
+  extern __shared__ __attribute__((aligned(16))) char smem_all[];
+  char* smem = smem_all + 4 * kAWave;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
-  const int wave = (tid / kWave) & 3;    // which 16 of the block's 64 rows
-  const int kgroup = tid / (4 * kWave);  // which part of the block's K slice
+  const int wave = tid / kWave;          // which 16 of the block's 64 rows
+  char* mine = smem_all + wave * kAWave;
   const int r16 = lane & 15;
   const int g = lane >> 4;
   const int k = p.k;
@@ -65,21 +65,21 @@ __global__ void __launch_bounds__(256 * KG) gemm_skinny_kernel(SkinnyParams p) {
   const int split = blockIdx.x - tile * p.splits;
   const int k_begin = split * p.kslice;
   const int k_end = min(k, k_begin + p.kslice);
-  // this wave's part of the slice: whole chunks
-  const int sub = ((p.kslice / KG + kSkinnyChunk - 1) / kSkinnyChunk) * kSkinnyChunk;
-  const int kw_begin = k_begin + kgroup * sub;
-  const int kw_end = min(k_end, kw_begin + sub);
+  const int kw_begin = k_begin, kw_end = k_end;
   const int xrow_bytes = p.xk * 2 + 16;   // 16 bytes of padding: rows start 4 banks apart
 
-  // the row of w this lane streams, and the output column it stands for
-  int wrow;
-  if (GATE) {
-    const int col = tile * 32 + (wave & 1) * 16 + r16;
-    wrow = min(col, p.inter - 1) + (wave >= 2 ? p.inter : 0);
-  } else {
-    wrow = min(tile * kSkinnyRows + wave * 16 + r16, p.n - 1);
-  }
-  const bf16_t* wp = p.w + (size_t)wrow * k + 8 * g;
+  // row j (0..15) of this wave in w
+  auto w_row = [&](int j) -> int {
+    if (GATE) {
+      const int col = tile * 32 + (wave & 1) * 16 + j;
+      return min(col, p.inter - 1) + (wave >= 2 ? p.inter : 0);
+    }
+    return min(tile * kSkinnyRows + wave * 16 + j, p.n - 1);
+  };
+  // load (rg, s) of a shot: this lane reads 16 bytes of row 4 rg + g at k 128 s + 8 r16
+  const bf16_t* wrow[4];
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg) wrow[rg] = p.w + (size_t)w_row(4 * rg + g) * k + 8 * r16;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
   f32x4 acc[MT];
@@ -89,19 +89,22 @@ __global__ void __launch_bounds__(256 * KG) gemm_skinny_kernel(SkinnyParams p) {
 #pragma unroll
   for (int t = 0; t < MT; ++t) xrow[t] = min(16 * t + r16, p.m - 1) * xrow_bytes + 16 * g;
 
-  bf16x8 a_next[U];
-  auto load_a = [&](int kc) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int kk = kc + 32 * u;
-      a_next[u] = (kk + 8 * g < k) ? *reinterpret_cast<const bf16x8*>(wp + kk) : zero;
-    }
-  };
-  const int nch = kw_begin < kw_end ? (kw_end - kw_begin + kSkinnyChunk - 1) / kSkinnyChunk : 0;
-  if (nch) load_a(kw_begin);
-
   for (int x0 = k_begin; x0 < k_end; x0 += p.xk) {
     const int x1 = min(k_end, x0 + p.xk);
+    // this wave's first shot in [x0, x1): its loads go out before x is staged
+    int kc = max(x0, kw_begin);
+    const int kc_end = min(x1, kw_end);
+    bf16x8 a[16];
+    auto load_shot = [&](int at) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int kk = at + 128 * (i >> 2);
+        a[i] = (kk + 8 * r16 < k) ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[i & 3] + kk))
+                                  : zero;
+      }
+    };
+    if (kc < kc_end) load_shot(kc);
+
     const int pieces = (x1 - x0 + 7) / 8;    // 16-byte pieces per row
     if (x0 != k_begin) __syncthreads();      // the previous slice of x has been read
     for (int q = tid; q < p.m * pieces; q += THREADS) {
@@ -110,57 +113,55 @@ __global__ void __launch_bounds__(256 * KG) gemm_skinny_kernel(SkinnyParams p) {
       const bf16x8 v = kk < k ? *reinterpret_cast<const bf16x8*>(p.x + (size_t)row * k + kk) : zero;
       *reinterpret_cast<bf16x8*>(smem + row * xrow_bytes + piece * 16) = v;
     }
-    // a chunk that reaches beyond K reads pieces the loop above did not write: zero them
+    // a shot that reaches beyond K reads pieces the loop above did not write: zero them
     const int padded = ((x1 - x0 + kSkinnyChunk - 1) / kSkinnyChunk) * (kSkinnyChunk / 8);
     for (int q = tid; q < p.m * (padded - pieces); q += THREADS) {
       const int row = q / (padded - pieces), piece = pieces + q - row * (padded - pieces);
       *reinterpret_cast<bf16x8*>(smem + row * xrow_bytes + piece * 16) = zero;
     }
     __syncthreads();
-    for (int kc = max(x0, kw_begin); kc < min(x1, kw_end); kc += kSkinnyChunk) {
-      bf16x8 a[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) a[u] = a_next[u];
-      if (kc + kSkinnyChunk < kw_end) load_a(kc + kSkinnyChunk);
+
+    for (; kc < kc_end; kc += kSkinnyChunk) {
       const char* xb = smem + (kc - x0) * 2;
 #pragma unroll
-      for (int u = 0; u < U; ++u)
+      for (int s4 = 0; s4 < 4; ++s4) {
+        // a quarter of the shot into the operand layout through the wave's own LDS area
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-          const bf16x8 bv = *reinterpret_cast<const bf16x8*>(xb + xrow[t] + 64 * u);
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc[t], 0, 0, 0);
+        for (int rg = 0; rg < 4; ++rg)
+          *reinterpret_cast<bf16x8*>(mine + (4 * rg + g) * kARow + r16 * 16) = a[4 * s4 + rg];
+        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the area is this wave's alone, no block barrier
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const bf16x8 av = *reinterpret_cast<const bf16x8*>(mine + r16 * kARow + u * 64 + g * 16);
+#pragma unroll
+          for (int t = 0; t < MT; ++t) {
+            const bf16x8 bv = *reinterpret_cast<const bf16x8*>(xb + xrow[t] + 64 * (4 * s4 + u));
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc[t], 0, 0, 0);
+          }
         }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+      }
+      if (kc + kSkinnyChunk < kc_end) load_shot(kc + kSkinnyChunk);
     }
   }
 
-  // ---- the block's float32 tile [m][64] through LDS, one per K group, added in group order:
-  //      lane holds rows m = 16 t + r16, columns 16 wave + 4 g + i
+  // ---- the block's float32 tile [m][64] through LDS: lane holds rows m = 16 t + r16, columns 16 wave + 4 g + i
   __syncthreads();
-  float* tile_f = reinterpret_cast<float*>(smem);   // [KG][m][65], then [m][65]
-  const int tile_floats = p.m * (kSkinnyRows + 1);
+  float* tile_f = reinterpret_cast<float*>(smem);   // [m][65]
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = 16 * t + r16;
     if (m < p.m) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        tile_f[kgroup * tile_floats + m * (kSkinnyRows + 1) + 16 * wave + 4 * g + i] = acc[t][i];
+      for (int i = 0; i < 4; ++i) tile_f[m * (kSkinnyRows + 1) + 16 * wave + 4 * g + i] = acc[t][i];
     }
   }
   __syncthreads();
-  if (KG > 1) {
-    for (int item = tid; item < p.m * kSkinnyRows; item += THREADS) {
-      const int at = (item >> 6) * (kSkinnyRows + 1) + (item & 63);
-      float v = tile_f[at];
-#pragma unroll
-      for (int kg = 1; kg < KG; ++kg) v += tile_f[kg * tile_floats + at];
-      tile_f[at] = v;
-    }
-    __syncthreads();
-  }
 
   if (p.splits > 1) {
-    float* mine = p.partial + (size_t)split * p.m * p.n;
+    float* out_slice = p.partial + (size_t)split * p.m * p.n;
     for (int item = tid; item < p.m * kSkinnyRows; item += THREADS) {
       const int m = item >> 6, c = item & 63;
       int col;
@@ -172,7 +173,7 @@ __global__ void __launch_bounds__(256 * KG) gemm_skinny_kernel(SkinnyParams p) {
         col = tile * kSkinnyRows + c;
         if (col >= p.n) continue;
       }
-      mine[(size_t)m * p.n + col] = tile_f[m * (kSkinnyRows + 1) + c];
+      out_slice[(size_t)m * p.n + col] = tile_f[m * (kSkinnyRows + 1) + c];
     }
     return;
   }
@@ -215,29 +216,18 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, const fl
 
 static int skinny_tiles(int n, int gate) { return gate ? (n + 31) / 32 : (n + kSkinnyRows - 1) / kSkinnyRows; }
 
-// How K is cut between blocks (slices a multiple of 512) and inside a block.
+// How K is cut between blocks: slices a multiple of 512.  Measured on an MI355X with the Qwen3-8B
+// products: narrow products (under 256 row tiles) run best with about 512 blocks, wide ones (gate/up,
+// head) with four slices.
 static SkinnyPlan skinny_plan(int m, int tiles, int k) {
   SkinnyPlan plan{};
   const int units = (k + 511) / 512;
-  if (tiles >= 256) {
-    // wide: sixteen waves a block, four K groups; the block's whole x slice sits in LDS, two blocks a CU
-    // where 80 KB hold it, else one
-    plan.kgroups = 4;
-    int cap = ((80 * 1024 / m - 16) / 2) / 1024 * 1024;
-    if (cap < 1024) cap = ((144 * 1024 / m - 16) / 2) / 1024 * 1024;   // m <= 64: at least 1024
-    plan.kslice = min(units * 512, cap);
-    plan.splits = (k + plan.kslice - 1) / plan.kslice;
-    plan.xk = ((plan.kslice + kSkinnyChunk - 1) / kSkinnyChunk) * kSkinnyChunk;
-    return plan;
-  }
-  // narrow: four waves a block and enough slices to keep about a thousand blocks in flight
-  plan.kgroups = 1;
-  int s = (1024 + tiles - 1) / tiles;
+  int s = tiles >= 256 ? 4 : (512 + tiles - 1) / tiles;
   s = max(1, min(s, min(units, 32)));
   const int per = (units + s - 1) / s;           // units of 512 per slice
   plan.kslice = per * 512;
   plan.splits = (units + per - 1) / per;
-  int cap = (kSkinnyLds - 64) / m / 2 - 8;       // k elements of one row of x that fit
+  int cap = (kSkinnyLds - 4 * kAWave - 64) / m / 2 - 8;   // k elements of one row of x that fit
   cap = max(kSkinnyChunk, cap / kSkinnyChunk * kSkinnyChunk);
   plan.xk = min(plan.kslice, cap);
   return plan;
@@ -275,29 +265,24 @@ ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias
   if (p.splits > 1 ? partial == nullptr : y == nullptr) return ATOM_BAD_SHAPE;
   const long blocks = (long)p.tiles * p.splits;
   if (blocks > 0x7fffffffL) return ATOM_TOO_LARGE;
-  const size_t lds = max((size_t)m * (p.xk * 2 + 16), (size_t)plan.kgroups * m * (kSkinnyRows + 1) * 4);
+  const size_t lds = (size_t)4 * kAWave + max((size_t)m * (p.xk * 2 + 16), (size_t)m * (kSkinnyRows + 1) * 4);
   const int mt = (m + 15) / 16;
-  const bool wide = plan.kgroups == 4;
-  // the wide kernels may need more LDS than a launch gets by default: allow it once per kernel
-#define GO_ONE(MTV, G, KGV)                                                                                   \
-  do {                                                                                                        \
-    if (KGV > 1) {                                                                                            \
-      static bool allowed = false;                                                                            \
-      if (!allowed) {                                                                                         \
-        if (hipFuncSetAttribute((const void*)gemm_skinny_kernel<MTV, G, KGV>,                                 \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)        \
-          return ATOM_LAUNCH_FAILED;                                                                          \
-        allowed = true;                                                                                       \
-      }                                                                                                       \
-    }                                                                                                         \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MTV, G, KGV>), dim3(blocks), dim3(256 * KGV), lds, stream, p);     \
+  // 64 rows of x need a little more LDS than a launch gets by default: allow it once per kernel
+#define GO_ONE(MTV, G)                                                                                   \
+  do {                                                                                                   \
+    static bool allowed = false;                                                                         \
+    if (!allowed) {                                                                                      \
+      if (hipFuncSetAttribute((const void*)gemm_skinny_kernel<MTV, G>,                                   \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess)      \
+        return ATOM_LAUNCH_FAILED;                                                                       \
+      allowed = true;                                                                                    \
+    }                                                                                                    \
+    hipLaunchKernelGGL((gemm_skinny_kernel<MTV, G>), dim3(blocks), dim3(256), lds, stream, p);           \
   } while (0)
-#define GO(MTV)                                  \
-  do {                                           \
-    if (gate && wide) GO_ONE(MTV, true, 4);      \
-    else if (gate) GO_ONE(MTV, true, 1);         \
-    else if (wide) GO_ONE(MTV, false, 4);        \
-    else GO_ONE(MTV, false, 1);                  \
+#define GO(MTV)                      \
+  do {                               \
+    if (gate) GO_ONE(MTV, true);     \
+    else GO_ONE(MTV, false);         \
   } while (0)
   switch (mt) {
     case 1: GO(1); break;
