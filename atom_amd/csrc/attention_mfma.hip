@@ -151,16 +151,33 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
     s16x4 k16[KX32 ? 1 : KCH];
     s16x4 v[DT];
   };
+  // Head sizes whose key rows are a whole number of 16-byte pieces per wave load (32, 64, 128, 256) are
+  // read in whole cache lines: piece q = 64 j + lane of the block is 8 elements of key q / (D / 8), and the
+  // block then goes through a small LDS area of the wave to reach the operand layout.
+  constexpr bool KROWS = KX32 && (D == 32 || D == 64 || D == 128 || D == 256);
+  constexpr int KLDS = D * 2 + 16;   // LDS bytes of a key row: rows start 4 banks apart
+  __shared__ __attribute__((aligned(16))) char klds[KROWS ? 16 * KLDS : 16];
   auto load_block = [&](int k0, KVBlock& blk) {
     // this lane's key row is k0 + r16 (clamped into the context for addressing)
     const int krow = min(k0 + r16, ke - 1);
     const int kpage = table[krow / ps];
     const bf16_t* kptr = p.k_cache + (((size_t)kpage * p.hkv + kvh) * ps + (krow % ps)) * D;
+    if (KROWS) {
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) {
+        const int q = 64 * j + lane;
+        const int row = min(k0 + q / (D / 8), ke - 1);
+        const int page = table[row / ps];
+        blk.k32[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(
+            p.k_cache + (((size_t)page * p.hkv + kvh) * ps + (row % ps)) * D + (q % (D / 8)) * 8));
+      }
+    }
     // this lane's V keys are k0 + 4g .. + 3, of output rows d = 16 t + r16
     const int vkey = min(k0 + 4 * g, ((ke - 1) & ~3));
     const int vpage = table[vkey / ps];
     const bf16_t* vptr = p.v_cache + (((size_t)vpage * p.hkv + kvh) * D + r16) * (size_t)ps + (vkey % ps);
-    if (KX32) {
+    if (KROWS) {
+    } else if (KX32) {
 #pragma unroll
       for (int j = 0; j < KCH; ++j) blk.k32[j] = *reinterpret_cast<const bf16x8*>(kptr + 32 * j + 8 * g);
     } else {
@@ -178,7 +195,23 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
     f32x4 s[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) s[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (KX32) {
+    if (KROWS) {
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) {
+        const int q = 64 * j + lane;
+        *reinterpret_cast<bf16x8*>(klds + (q / (D / 8)) * KLDS + (q % (D / 8)) * 16) = cur.k32[j];
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0); the block is one wave
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(klds + r16 * KLDS + 64 * j + 16 * g);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) s[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q32[rt][j], s[rt], 0, 0, 0);
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_wave_barrier();
+    } else if (KX32) {
 #pragma unroll
       for (int j = 0; j < KCH; ++j)
 #pragma unroll
