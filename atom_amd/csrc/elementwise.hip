@@ -337,9 +337,10 @@ __global__ void qk_norm_rope_kv_write_kernel(
     const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ slots,
-    int hq, int hkv, int d, int rotary_dim, int page_size, float eps, int write_kv, SplitSum xsum) {
+    int hq, int hkv, int d, int rotary_dim, int page_size, float eps, int write_kv, SplitSum xsum,
+    int head_begin) {
   const int t = blockIdx.x;
-  const int head = blockIdx.y;  // 0..hq-1 q, then hkv k heads, then hkv v heads
+  const int head = blockIdx.y + head_begin;  // 0..hq-1 q, then hkv k heads, then hkv v heads
   const int lane = threadIdx.x;
   const int row_width = (hq + 2 * hkv) * d;
   const T* src = qkv + (size_t)t * row_width + (size_t)head * d;
@@ -429,6 +430,68 @@ __global__ void qk_norm_rope_kv_write_kernel(
   }
 }
 
+// The q and k heads of many tokens, when the whole head is rotated and the input is a tensor: sixteen lanes
+// per (token, head), each with D / 16 consecutive elements (vector loads and stores); the rotation partner
+// of a lane is 8 lanes away.  256 threads are 16 (token, head) pairs.
+template <typename T, int E>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_vec_kernel(const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache,
+                        const float* __restrict__ q_weight, const float* __restrict__ k_weight,
+                        const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+                        const int* __restrict__ positions, const int* __restrict__ slots, int tokens, int hq, int hkv,
+                        int page_size, float eps, int write_kv) {
+  constexpr int D = 16 * E;
+  const int pair = blockIdx.x * 16 + threadIdx.x / 16;
+  const int i = threadIdx.x & 15;
+  const int heads = hq + hkv;
+  const bool live = pair < tokens * heads;
+  const int t = live ? pair / heads : 0;
+  const int head = live ? pair - t * heads : 0;
+  const bool is_q = head < hq;
+  const size_t row_width = (size_t)(hq + 2 * hkv) * D;
+  constexpr int ALIGN = sizeof(T) * E < 16 ? sizeof(T) * E : 16;
+  T raw[E];
+  __builtin_memcpy(raw, __builtin_assume_aligned(qkv + (size_t)t * row_width + (size_t)head * D + E * i, ALIGN),
+                   sizeof(raw));
+  float x[E];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    x[e] = to_f32(raw[e]);
+    ss += x[e] * x[e];
+  }
+  const float* weight = is_q ? q_weight : k_weight;
+  if (weight) {
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 16);
+    const float inv = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+    for (int e = 0; e < E; ++e) x[e] = x[e] * inv * weight[E * i + e];
+  }
+  const int pos = positions[t];
+  const float* cs = cos_table + (size_t)pos * (D / 2) + E * (i & 7);
+  const float* sn = sin_table + (size_t)pos * (D / 2) + E * (i & 7);
+  T out[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const float other = __shfl_xor(x[e], 8, 16);
+    const float c = cs[e], sv = sn[e];
+    out[e] = from_f32<T>(i < 8 ? x[e] * c - other * sv : x[e] * c + other * sv);
+  }
+  if (!live) return;
+  T* dst;
+  if (is_q) {
+    dst = q_out + ((size_t)t * hq + head) * D + E * i;
+  } else {
+    if (!write_kv) return;
+    const int slot = slots[t];
+    if (slot < 0) return;
+    const int page = slot / page_size, off = slot - page * page_size;
+    dst = k_cache + (((size_t)page * hkv + (head - hq)) * page_size + off) * (size_t)D + E * i;
+  }
+  __builtin_memcpy(__builtin_assume_aligned(dst, ALIGN), out, sizeof(out));
+}
+
 ATOM_EXPORT int atom_qk_norm_rope_kv_write(
     const void* qkv, void* q_out, void* k_cache, void* v_cache, const float* q_weight, const float* k_weight,
     const float* cos_table, const float* sin_table, const int* positions, const int* slots, int dtype,
@@ -442,10 +505,32 @@ ATOM_EXPORT int atom_qk_norm_rope_kv_write(
   if (write_kv && (!k_cache || !v_cache || !slots)) return ATOM_BAD_SHAPE;
   if (hq + 2 * hkv > 65535) return ATOM_TOO_LARGE;
   if (tokens == 0) return ATOM_OK;
-  dim3 grid(tokens, hq + 2 * hkv), block(kWave);
+  int head_begin = 0;
+  const long pairs = (long)tokens * (hq + hkv);
+  if (!x_partial && tokens >= 32 && rotary_dim == d && d % 16 == 0 && d <= 256 && (d & (d - 1)) == 0 &&
+      pairs / 16 < 0x7fffffffL && (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache) & 31) == 0) {
+    // many tokens: q and k heads through the vector kernel, the value heads through the general one
+    const dim3 vgrid((unsigned)((pairs + 15) / 16)), vblock(256);
+#define LAUNCH_ROPE(EE)                                                                                          \
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((qk_norm_rope_vec_kernel<T, EE>), vgrid, vblock, 0, stream,      \
+                                                 (const T*)qkv, (T*)q_out, (T*)k_cache, q_weight, k_weight,      \
+                                                 cos_table, sin_table, positions, slots, tokens, hq, hkv,        \
+                                                 page_size, eps, write_kv))
+    switch (d / 16) {
+      case 1: LAUNCH_ROPE(1); break;
+      case 2: LAUNCH_ROPE(2); break;
+      case 4: LAUNCH_ROPE(4); break;
+      case 8: LAUNCH_ROPE(8); break;
+      default: LAUNCH_ROPE(16); break;
+    }
+#undef LAUNCH_ROPE
+    if (!write_kv) return launch_status();
+    head_begin = hq + hkv;
+  }
+  dim3 grid(tokens, hq + 2 * hkv - head_begin), block(kWave);
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<T>), grid, block, 0, stream,
                                                  (const T*)qkv, (T*)q_out, (T*)k_cache, (T*)v_cache, q_weight,
                                                  k_weight, cos_table, sin_table, positions, slots, hq, hkv, d,
-                                                 rotary_dim, page_size, eps, write_kv, xsum));
+                                                 rotary_dim, page_size, eps, write_kv, xsum, head_begin));
   return launch_status();
 }

@@ -125,16 +125,18 @@ def test_linear_bf16_library_path():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hq,hkv,d,rot,page", [(4, 2, 16, 16, 16), (6, 3, 32, 32, 8), (5, 5, 48, 24, 4),
-                                              (8, 1, 128, 128, 32), (3, 1, 80, 0, 16)])
+                                              (8, 1, 128, 128, 32), (3, 1, 80, 0, 16), (5, 2, 64, 64, 16),
+                                              (2, 1, 256, 256, 8), (3, 3, 96, 96, 16)])
 @pytest.mark.parametrize("norm", [True, False])
-def test_qk_norm_rope_kv_write(dtype, hq, hkv, d, rot, page, norm):
-    tokens, pages, max_pos = 11, 6, 50
+@pytest.mark.parametrize("tokens", [11, 45])   # 32 tokens and more take the vector kernel where it applies
+def test_qk_norm_rope_kv_write(dtype, hq, hkv, d, rot, page, norm, tokens):
+    pages, max_pos = -(-64 // page), 50
     qkv = rnd((tokens, (hq + 2 * hkv) * d), dtype, 16, 2.0)
     qw = 1 + rnd((d,), torch.float32, 17, 0.2) if norm else None
     kw = 1 + rnd((d,), torch.float32, 18, 0.2) if norm else None
     ang = torch.outer(torch.arange(max_pos, dtype=torch.float32), 1.0 / (1e4 ** (torch.arange(0, max(rot, 2), 2) / max(rot, 2))))
     cos, sin = ang.cos().contiguous(), ang.sin().contiguous()
-    positions = torch.tensor([3, 4, 5, 0, 1, 49, 20, 21, 22, 23, 7], dtype=torch.int32)
+    positions = torch.tensor(([3, 4, 5, 0, 1, 49, 20, 21, 22, 23, 7] * 5)[:tokens], dtype=torch.int32)
     perm = torch.randperm(pages * page, generator=torch.Generator().manual_seed(19))[:tokens].to(torch.int32)
     slots = perm.clone()
     slots[4] = -1   # a padding row writes nothing
