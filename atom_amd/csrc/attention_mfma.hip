@@ -41,7 +41,7 @@ struct AttnParams {
   const int* tiles;       // prefill: [num_tiles, 2] = (request, first row of the tile within its tokens)
   float* ws_o;            // decode: [seqs, Hq, parts, D]
   float* ws_ml;           // decode: [seqs, Hq, parts, 2]
-  int max_blocks, hq, hkv, page_size, window, seq_offset, parts;
+  int max_blocks, hq, hkv, page_size, window, seq_offset, parts, num_tiles;
   float scale_log2;       // softmax scale * log2(e)
 };
 
@@ -397,7 +397,11 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
   const int group = p.hq / p.hkv;
   const int ps = p.page_size;
 
-  const int tile = blockIdx.x;
+  // A block takes two tiles, one after the other: the host lists tiles with the most keys first, so tile b and
+  // tile n - 1 - b together are about the same work for every b, and all blocks finish together.
+  for (int pass = 0; pass < 2; ++pass) {
+  const int tile = pass == 0 ? (int)blockIdx.x : p.num_tiles - 1 - (int)blockIdx.x;
+  if (pass == 1 && tile <= (int)blockIdx.x) break;
   const int seq = p.tiles[2 * tile];
   const int row_start = p.tiles[2 * tile + 1];
   const int head = blockIdx.y * GH + (wave % GH);
@@ -580,6 +584,7 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
       *reinterpret_cast<bf16x4*>(dst + 16 * t + 4 * g) = o;
     }
   }
+  }   // the two tiles of the block
 }
 
 // Query tokens per block of the tiled prefill kernel for this head size, page size and group, or 0
@@ -595,8 +600,8 @@ static int launch_prefill_tiled(const AttnParams& p, int num_tiles, int rows_per
   const int group = p.hq / p.hkv;
   const int gh = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
   if (rows_per_tile != 32 * (4 / gh)) return ATOM_BAD_SHAPE;
-  dim3 grid(num_tiles, p.hq / gh), block(256);
-  constexpr int TK = 32;   // 64 needs so many registers that one block a CU is left, which is slower
+  dim3 grid((num_tiles + 1) / 2, p.hq / gh), block(256);
+  constexpr int TK = D <= 128 ? 64 : 32;
   if (gh == 4) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 4, TK>), grid, block, 0, stream, p);
   else if (gh == 2) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 2, TK>), grid, block, 0, stream, p);
   else hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 1, TK>), grid, block, 0, stream, p);
@@ -673,6 +678,7 @@ ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const
   p.out = (bf16_t*)out; p.cu_q = cu_q; p.ctx_lens = ctx_lens; p.block_tables = block_tables; p.tiles = tiles;
   p.ws_o = nullptr; p.ws_ml = nullptr; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
   p.window = window; p.seq_offset = 0; p.parts = 1; p.scale_log2 = scale * 1.4426950408889634f;
+  p.num_tiles = num_tiles;
   if (tiled) {   // tiles of atom_attention_prefill_tile_rows() tokens for the kernel with shared key tiles
     if (!atom_attention_prefill_tile_rows(d, page_size, hq / hkv)) return ATOM_UNSUPPORTED;
     switch (d) {
