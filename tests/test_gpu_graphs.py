@@ -34,16 +34,19 @@ def test_graph_cuts_match_plain(which, cut, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_replays_agree_with_eager(dtype):
-    """Three requests decode together through one graph (bucket 4, one padding row) for 12 steps; in
-    between, another request runs eager prompt portions.  An eager engine runs the same steps."""
+@pytest.mark.parametrize("live,bucket", [(3, 4), (27, 32)])
+def test_replays_agree_with_eager(dtype, live, bucket):
+    """Requests decode together through one graph (with padding rows) for 12 steps; in between, another
+    request runs eager prompt portions.  An eager engine runs the same steps.  With 27 rows the bfloat16
+    products inside the graph are the BLAS library's, with 3 the engine's own."""
     which = "C"
-    prompts = {f"p{k}": random_ids(which, n, 40 + k) for k, n in enumerate([33, 70, 150])}
+    prompts = {f"p{k}": random_ids(which, n, 40 + k) for k, n in enumerate(([33, 70, 150] * 9)[:live])}
     tails = {rid: random_ids(which, 12, 60 + k) for k, rid in enumerate(prompts)}
     other = random_ids(which, 200, 99)
 
     def run(graph_sizes):
-        core = make_core(which, dtype, gpu_ops(), "cuda:0", num_pages=64, page_size=16, graph_sizes=graph_sizes)
+        core = make_core(which, dtype, gpu_ops(), "cuda:0", num_pages=64 + 12 * live, page_size=16,
+                         max_num_seqs=max(live + 1, bucket), graph_sizes=graph_sizes)
         for rid, ids in prompts.items():
             core.step([StepEntry(rid, ids, [])])
         outs = []
@@ -55,7 +58,7 @@ def test_replays_agree_with_eager(dtype):
         return outs, core
 
     eager, _ = run(None)
-    graphed, core = run([4])
+    graphed, core = run([bucket])
     assert core.graphs.replays == 12
     scale = max(float(e.abs().max()) for e in eager)
     tol = 1e-5 if dtype == "float32" else 2e-2
