@@ -175,9 +175,8 @@ class Scheduler:
 
         # ---- running requests that decode: one token each
         for seq in list(self.running):
+            # a request preempted earlier in this loop is WAITING by now
             if seq.status != SequenceStatus.RUNNING or seq.is_partial_prefill or seq.id in scheduled:
-                continue
-            if seq not in self.running:   # preempted meanwhile
                 continue
             if len(batch.items) >= self.max_num_seqs or batched + 1 > self.max_num_batched_tokens:
                 break
@@ -199,7 +198,7 @@ class Scheduler:
 
         # ---- unfinished prompts among the running requests
         for seq in list(self.running):
-            if not seq.is_partial_prefill or seq.id in scheduled or seq not in self.running:
+            if not seq.is_partial_prefill or seq.id in scheduled or seq.status != SequenceStatus.RUNNING:
                 continue
             if len(batch.items) >= self.max_num_seqs:
                 break
