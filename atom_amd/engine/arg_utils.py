@@ -48,6 +48,7 @@ class EngineArgs:
     cudagraph_capture_sizes: str = "[1,2,4,8,16,32,48,64,128,256]"
     load_dummy: str | None = None
     torch_profiler_dir: str | None = None
+    mark_trace: bool = False
     hf_overrides: dict | None = None
     num_kvcache_blocks: int = -1
     dtype: str = "bf16"
@@ -76,6 +77,8 @@ class EngineArgs:
         parser.add_argument("--load-dummy", type=str, nargs="?", const="random", default=None,
                             help="Skip the checkpoint: seeded random weights.")
         parser.add_argument("--torch-profiler-dir", type=str, default=None, help="Write a torch.profiler trace here.")
+        parser.add_argument("--mark-trace", action="store_true",
+                            help="Name every operation's kernels in profiler traces (record_function spans).")
         parser.add_argument("--hf-overrides", type=json.loads, default=None, help="JSON dict of config.json overrides.")
         parser.add_argument("--num-kvcache-blocks", type=int, default=-1, help="Cache pages (-1: from free memory).")
         parser.add_argument("--dtype", choices=["bf16", "bfloat16", "fp32", "float32"], default="bf16",

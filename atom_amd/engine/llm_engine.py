@@ -48,6 +48,8 @@ class LLMEngine:
             from ..kernels.hip import HipKernels
 
             ops = HipKernels(cfg.device)
+        if cfg.mark_trace and hasattr(ops, "mark_trace"):
+            ops.mark_trace()
         self.ops = ops
         source = weight_source
         if source is None and cfg.load_dummy:

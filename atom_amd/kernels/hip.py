@@ -138,6 +138,28 @@ class HipKernels:
             self._ws[name] = t
         return t
 
+    # the span names of the operations in a profiler trace, the reference's where it has one
+    # (atom/model_ops/attention_mha.py:199, 483, 729: "rope_cache", "paged_attention_*", "prefill_attention")
+    _SPANS = {"embedding": "embedding", "rmsnorm": "rmsnorm", "silu_mul": "silu_mul",
+              "qk_norm_rope_kv_write": "rope_cache", "paged_attention": "paged_attention",
+              "linear": "linear", "linear_silu": "linear_silu", "sample": "sample"}
+
+    def mark_trace(self) -> None:
+        """Wraps every operation of this object in a ``torch.profiler.record_function`` span, so that a
+        profiler trace shows which kernels belong to which operation (the reference's ``--mark-trace``,
+        atom/utils/decorators.py:232-257, in its record_function form).  Off by default: a span costs
+        host time in every call."""
+        for method, span in self._SPANS.items():
+            inner = getattr(self, method)
+            if getattr(inner, "_marked", False):
+                continue
+
+            def marked(*args, _inner=inner, _span=span, **kwargs):
+                with torch.profiler.record_function(_span):
+                    return _inner(*args, **kwargs)
+            marked._marked = True
+            setattr(self, method, marked)
+
     def decode_parts(self, seqs: int, hkv: int, max_context: int) -> int:
         """Over how many waves a decode row's keys are split: enough waves to fill the chip,
         at least 64 keys each."""

@@ -111,8 +111,10 @@ def test_cli_flags_in_both_spellings():
     parser = FlexibleArgumentParser()
     EngineArgs.add_cli_args(parser)
     a = EngineArgs.from_cli_args(parser.parse_args(["--model", "m", "--max-model-len", "99", "--block_size=32",
-                                                    "--no-enable-chunked-prefill", "--max_num_seqs", "7"]))
+                                                    "--no-enable-chunked-prefill", "--max_num_seqs", "7",
+                                                    "--mark-trace"]))
     assert (a.model, a.max_model_len, a.block_size, a.enable_chunked_prefill, a.max_num_seqs) == ("m", 99, 32, False, 7)
+    assert a.mark_trace and not EngineArgs(model="m").mark_trace
     kw = a._get_engine_kwargs()
     assert kw["kv_cache_block_size"] == 32 and "block_size" not in kw
     assert kw["cudagraph_capture_sizes"][:3] == [1, 2, 4]

@@ -126,6 +126,24 @@ def test_stop_on_eos_and_logprobs():
     assert rejected["finish_reason"].startswith("unschedulable")
 
 
+def test_mark_trace_names_the_operations_in_a_profile():
+    """With mark_trace the steps' spans hold one span per operation, and the tokens do not change."""
+    from atom_amd.kernels.hip import HipKernels
+
+    prompt = random_ids("B", 20, 5)
+    sp = SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True)
+    plain_run = engine("B", "bf16").generate([prompt], sp)[0]["token_ids"]
+    llm = LLMEngine(tiny_folder("B"), dtype="bf16", ops=HipKernels("cuda:0"), mark_trace=True, enforce_eager=True,
+                    kv_cache_block_size=PAGE["B"], num_kvcache_blocks=64, max_num_seqs=4)
+    with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CPU]) as prof:
+        marked_run = llm.generate([prompt], sp)[0]["token_ids"]
+    assert marked_run == plain_run
+    names = {e.key for e in prof.key_averages()}
+    for span in ("rope_cache", "paged_attention", "rmsnorm", "linear", "linear_silu", "embedding", "sample"):
+        assert span in names, (span, sorted(n for n in names if not n.startswith("aten::")))
+    assert any(n.startswith("prefill[bs=1 tok=20") for n in names) and any(n.startswith("decode[bs=1") for n in names)
+
+
 def test_command_line():
     cmd = [sys.executable, "-m", "atom_amd.examples.simple_inference", "--model", tiny_folder("A"), "--temperature", "0",
            "--max-tokens", "8", "--block_size", "16", "--num-kvcache-blocks", "32", "--max-num-seqs", "4", "--dtype", "fp32",
