@@ -171,6 +171,7 @@ class _Request:
     serial: int = 0           # unique per ``open``: a request id that is opened again gets a new one
     tokens: list[int] = field(default_factory=list)   # prefix cache: the tokens that are in the cache
     hashes: list[int] = field(default_factory=list)   # prefix cache: chained hash of every full page so far
+    unknown_at: int | None = None   # prefix cache: position of a token that ran before the host knew its value
 
 
 class CacheManager:
@@ -345,6 +346,8 @@ class CacheManager:
 
     def _publish(self, req: _Request, cached_after: int) -> None:
         page_size = self.groups[0].page_size
+        if req.unknown_at is not None:   # a page is named only once all its tokens are known
+            cached_after = min(cached_after, req.unknown_at)
         while len(req.hashes) < cached_after // page_size:
             idx = len(req.hashes)
             tokens = tuple(req.tokens[idx * page_size:(idx + 1) * page_size])
@@ -353,15 +356,20 @@ class CacheManager:
             for gi, pool in enumerate(self.pools):
                 pool.publish(req.tables[gi][idx], content_hash, tokens)
 
-    def commit(self, req_id, cached_after: int, tokens=None) -> None:
+    def commit(self, req_id, cached_after: int, tokens=None, last_unknown: bool = False) -> None:
         """After a step: ``cached_after`` tokens are in the cache (``tokens``: the ones this step ran,
-        which the prefix cache needs to name the pages they filled).  Pages of window groups that no
-        later query can see are given back."""
+        which the prefix cache needs to name the pages they filled; ``last_unknown``: the last of them
+        was taken from the device and its value comes later, through ``amend``).  Pages of window groups
+        that no later query can see are given back."""
         req = self._requests[req_id]
         req.fresh = False
         if self.prefix_caching:
             if tokens is None:
                 raise ValueError("the prefix cache needs the tokens of every step")
+            if last_unknown:
+                if req.unknown_at is not None:
+                    raise AssertionError(f"request {req_id!r}: a second token whose value is not known yet")
+                req.unknown_at = len(req.tokens) + len(tokens) - 1
             req.tokens.extend(int(t) for t in tokens)
             if len(req.tokens) != cached_after:
                 raise AssertionError(f"request {req_id!r}: {len(req.tokens)} tokens noted, {cached_after} in the cache")
@@ -375,6 +383,22 @@ class CacheManager:
                 if table[idx] >= 0:
                     self.pools[gi].give(table[idx])
                     table[idx] = -1
+
+    def awaited_position(self, req_id) -> int | None:
+        """The position whose token ``commit`` took as not yet known, if there is one."""
+        return self._requests[req_id].unknown_at
+
+    def amend(self, req_id, position: int, token: int) -> None:
+        """The value of the token at ``position``, which ``commit`` took as not yet known."""
+        if not self.prefix_caching:
+            return
+        req = self._requests[req_id]
+        if req.unknown_at != position:
+            raise AssertionError(f"request {req_id!r}: position {position} is not the one whose token is awaited "
+                                 f"({req.unknown_at})")
+        req.tokens[position] = int(token)
+        req.unknown_at = None
+        self._publish(req, len(req.tokens))
 
     def block_table(self, req_id, group: int) -> list[int]:
         return self._requests[req_id].tables[group]

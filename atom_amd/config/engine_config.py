@@ -28,6 +28,7 @@ class Config:
     load_dummy: str | None = None
     torch_profiler_dir: str | None = None
     mark_trace: bool = False
+    deferred_output: bool = True
     cudagraph_capture_sizes: list[int] = field(default_factory=lambda: [1, 2, 4, 8, 16, 32, 48, 64, 128, 256])
     hf_overrides: dict | None = None
     dtype: str = "bf16"

@@ -51,6 +51,29 @@ ATOM_EXPORT int atom_embedding(const void* table, int table_dtype, const int* id
   return launch_status();
 }
 
+// ------------------------------------------------------------------ token ids that are still on the device
+//
+// ids[t] = sampled[source[t]] where source[t] >= 0: a request that decodes takes the token the last step
+// sampled for it from the sampler's own output, so that the step can be launched before the host has
+// read that token.  Rows with source[t] < 0 keep the id the host wrote.
+
+__global__ void feed_tokens_kernel(int* __restrict__ ids, const int* __restrict__ source,
+                                   const int* __restrict__ sampled, int tokens, int num_sampled) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= tokens) return;
+  const int src = source[t];
+  if (src >= 0 && src < num_sampled) ids[t] = sampled[src];
+}
+
+ATOM_EXPORT int atom_feed_tokens(int* ids, const int* source, const int* sampled, int tokens, int num_sampled,
+                                 hipStream_t stream) {
+  if (tokens < 0 || num_sampled < 0) return ATOM_BAD_SHAPE;
+  if (tokens == 0) return ATOM_OK;
+  hipLaunchKernelGGL(feed_tokens_kernel, dim3((tokens + 255) / 256), dim3(256), 0, stream, ids, source, sampled,
+                     tokens, num_sampled);
+  return launch_status();
+}
+
 // ------------------------------------------------------------------ RMS norm
 //
 // mode 0: y = norm(x)                                   (residual untouched)

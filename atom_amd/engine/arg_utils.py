@@ -49,6 +49,7 @@ class EngineArgs:
     load_dummy: str | None = None
     torch_profiler_dir: str | None = None
     mark_trace: bool = False
+    deferred_output: bool = True
     hf_overrides: dict | None = None
     num_kvcache_blocks: int = -1
     dtype: str = "bf16"
@@ -79,6 +80,8 @@ class EngineArgs:
         parser.add_argument("--torch-profiler-dir", type=str, default=None, help="Write a torch.profiler trace here.")
         parser.add_argument("--mark-trace", action="store_true",
                             help="Name every operation's kernels in profiler traces (record_function spans).")
+        parser.add_argument("--deferred-output", action=argparse.BooleanOptionalAction, default=True,
+                            help="Launch the next decode step before the host has read the last one's tokens.")
         parser.add_argument("--hf-overrides", type=json.loads, default=None, help="JSON dict of config.json overrides.")
         parser.add_argument("--num-kvcache-blocks", type=int, default=-1, help="Cache pages (-1: from free memory).")
         parser.add_argument("--dtype", choices=["bf16", "bfloat16", "fp32", "float32"], default="bf16",

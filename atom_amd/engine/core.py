@@ -34,6 +34,10 @@ class StepEntry:
     tokens: list[int]
     want: list[int] = field(default_factory=list)   # places among ``tokens`` whose logits are wanted
     reserve: int | None = None                      # pages are held up to this length (admission)
+    # The entry's one token is row ``feed`` of ``EngineCore.sampled`` (what the last step's sampler wrote
+    # there) and is read on the device; ``tokens`` then holds a placeholder.  The reference feeds decode
+    # steps the same way (atom/model_ops/decode_input_ids.py:1-32, model_runner.py:553-560).
+    feed: int | None = None
 
 
 class EngineCore:
@@ -56,6 +60,8 @@ class EngineCore:
         self.max_positions = model.spec.max_positions
         self.steps_run = 0
         self._fresh_slots: list[int] = []      # slots claimed since the last step: zeroed before it runs
+        # where a sampler leaves its tokens when the next step is to read them on the device (StepEntry.feed)
+        self.sampled = torch.zeros(max(1, max_num_seqs), dtype=torch.int32, device=self.device)
         # decode-only steps replay a captured HIP graph per batch-size bucket (None: always eager)
         self.graphs = None
         if graph_sizes:
@@ -123,6 +129,9 @@ class EngineCore:
                 raise ValueError(f"request {e.req_id!r}: a step entry needs at least one token")
             if min(e.tokens) < 0 or max(e.tokens) >= vocab:
                 raise ValueError(f"request {e.req_id!r}: token id outside [0, {vocab})")
+            if e.feed is not None and (len(e.tokens) != 1 or not 0 <= e.feed < self.sampled.numel()):
+                raise ValueError(f"request {e.req_id!r}: a token read on the device must be the entry's only one "
+                                 f"and name one of the {self.sampled.numel()} sampled rows")
             if any(w < 0 or w >= len(e.tokens) for w in e.want):
                 raise ValueError(f"request {e.req_id!r}: a wanted place is outside its {len(e.tokens)} tokens")
             end = self.num_cached(e.req_id) + len(e.tokens)
@@ -157,9 +166,16 @@ class EngineCore:
 
         for e in entries:
             self.lengths[e.req_id] += len(e.tokens)
-            self.manager.commit(e.req_id, self.lengths[e.req_id], e.tokens if self.prefix_caching else None)
+            self.manager.commit(e.req_id, self.lengths[e.req_id], e.tokens if self.prefix_caching else None,
+                                last_unknown=e.feed is not None)
         self.steps_run += 1
         return logits
+
+    def resolve(self, req_id, position: int, token: int) -> None:
+        """Tells the cache's bookkeeping the value of a token that a step read on the device
+        (``StepEntry.feed``); a request that has ended meanwhile, or whose token no step has read, is skipped."""
+        if req_id in self.lengths and self.manager.awaited_position(req_id) == position:
+            self.manager.amend(req_id, position, token)
 
     def _build(self, entries: list[StepEntry], order: list[int]):
         mgr = self.manager
@@ -200,7 +216,13 @@ class EngineCore:
         # taller tiles for the prefill kernel whose waves share key tiles (its height depends on the layer)
         tall = {rows: tiles_of(rows) for rows in (32, 64, 128)} if max(q_lens) >= 32 else {}
 
-        pieces = [tokens, positions, token_seq, starts, context_lens, want_rows, tiles, *tall.values()]
+        feeds = any(e.feed is not None for e in entries)
+        feed = np.full(total if feeds else 0, -1, dtype=np.int32)
+        if feeds:
+            for i, e in enumerate(entries):
+                if e.feed is not None:
+                    feed[row_of_entry[i]] = e.feed
+        pieces = [tokens, positions, token_seq, starts, context_lens, want_rows, tiles, feed, *tall.values()]
         group_shapes = []
         for gi, g in enumerate(mgr.groups):
             tables = [mgr.block_table(entries[i].req_id, gi) for i in order]
@@ -227,9 +249,11 @@ class EngineCore:
         def view(k):
             return dev[offsets[k]:offsets[k] + pieces[k].size]
 
-        d_tokens, d_positions, d_token_seq, d_starts, d_ctx, d_want, d_tiles = (view(k) for k in range(7))
-        d_tall = {rows: view(7 + j).view(-1, 2) for j, rows in enumerate(tall)}
-        first_group = 7 + len(tall)
+        d_tokens, d_positions, d_token_seq, d_starts, d_ctx, d_want, d_tiles, d_feed = (view(k) for k in range(8))
+        if feeds:
+            self.ops.feed_tokens(d_tokens, d_feed, self.sampled)
+        d_tall = {rows: view(8 + j).view(-1, 2) for j, rows in enumerate(tall)}
+        first_group = 8 + len(tall)
         ctx = StepContext(ops=self.ops, dtype=self.dtype, device=self.device, num_tokens=total, num_seqs=num_seqs,
                           positions=d_positions, seq_starts=[int(s) for s in starts[:-1]], seq_lens=q_lens,
                           seq_cached=cached,

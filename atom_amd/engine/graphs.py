@@ -69,7 +69,7 @@ class DecodeGraphs:
     # ------------------------------------------------------------------ layout
 
     def _layout(self, size: int) -> tuple[dict[str, tuple[int, int]], int]:
-        pieces = [("tokens", size), ("positions", size), ("token_seq", size), ("starts", size + 1),
+        pieces = [("tokens", size), ("feed", size), ("positions", size), ("token_seq", size), ("starts", size + 1),
                   ("context_lens", size), ("want", size)]
         for gi, width in enumerate(self.widths):
             pieces += [(f"bt{gi}", size * width), (f"slots{gi}", size)]
@@ -94,6 +94,8 @@ class DecodeGraphs:
 
         tokens, positions, token_seq = view("tokens"), view("positions"), view("token_seq")
         tokens[:] = 0
+        feed = view("feed")
+        feed[:] = -1
         positions[:] = 0
         token_seq[:] = -1
         ctx_lens = view("context_lens")
@@ -102,6 +104,8 @@ class DecodeGraphs:
         view("want")[:] = np.arange(size, dtype=np.int32)
         for b, e in enumerate(entries):
             tokens[b] = e.tokens[0]
+            if e.feed is not None:
+                feed[b] = e.feed
             positions[b] = cached[b]
             token_seq[b] = b
             ctx_lens[b] = cached[b] + 1
@@ -149,7 +153,7 @@ class DecodeGraphs:
                 context_lens=view("context_lens"), num_seqs=size, num_tokens=size, max_q_len=1,
                 max_context_len=width * g.page_size, page_size=g.page_size, num_prefill=0, prefill_tiles=None)
             ctx.slot_mappings[gi] = view(f"slots{gi}")
-        return ctx, view("tokens"), view("want")
+        return ctx, view("tokens"), view("want"), view("feed")
 
     # ------------------------------------------------------------------ capture and replay
 
@@ -161,10 +165,11 @@ class DecodeGraphs:
         cap.dev = torch.zeros(max(total, 4), dtype=torch.int32, device=core.device)
         self._fill(cap, [], [])                       # all padding: the warm-up touches no cache slot
         cap.dev.copy_(cap.host)
-        ctx, tokens, want = self._context(cap)
+        ctx, tokens, want, feed = self._context(cap)
         stream = torch.cuda.Stream(device=core.device)
         stream.wait_stream(torch.cuda.current_stream(core.device))
         with torch.cuda.stream(stream):
+            core.ops.feed_tokens(tokens, feed, core.sampled)
             core.model.forward(ctx, tokens, core.storage.bindings, want)   # first-use allocations happen here
         stream.synchronize()
         if self.pool is None:
@@ -178,6 +183,8 @@ class DecodeGraphs:
         gc.disable()
         try:
             with torch.cuda.graph(cap.graph, pool=self.pool, stream=stream):
+                # rows whose token the last step's sampler left on the device take it from there
+                core.ops.feed_tokens(tokens, feed, core.sampled)
                 cap.logits = core.model.forward(ctx, tokens, core.storage.bindings, want)
         finally:
             if gc_was_enabled:

@@ -22,7 +22,7 @@ from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .core import TORCH_DTYPES, build_core, load_model
 from .scheduler import Scheduler
-from .sequence import Sequence
+from .sequence import Sequence, SequenceStatus
 
 logger = logging.getLogger("atom_amd")
 
@@ -35,6 +35,39 @@ def _load_tokenizer(path: str):
     from transformers import AutoTokenizer
 
     return AutoTokenizer.from_pretrained(path)
+
+
+class _Stage:
+    """Host memory (pinned where there is a GPU) that a step's sampled tokens and their log-probabilities
+    are copied into."""
+
+    def __init__(self, rows: int, pinned: bool):
+        self.pinned = pinned
+        self.grow(max(1, rows))
+
+    def grow(self, rows: int) -> None:
+        self.tokens = torch.zeros(rows, dtype=torch.int32, pin_memory=self.pinned)
+        self.logprobs = torch.zeros(rows, dtype=torch.float32, pin_memory=self.pinned)
+
+
+class _InFlight:
+    """A step that has been queued on the device and not yet read."""
+
+    def __init__(self, batch, finals, start: float):
+        self.batch = batch
+        self.finals = finals
+        self.start = start
+        self.tokens: torch.Tensor | None = None
+        self.logprobs: torch.Tensor | None = None
+        self.ready = torch.cuda.Event() if torch.cuda.is_available() else _NoEvent()
+
+
+class _NoEvent:
+    def record(self):
+        pass
+
+    def synchronize(self):
+        pass
 
 
 class LLMEngine:
@@ -73,6 +106,11 @@ class LLMEngine:
         self.sampler = Sampler(ops, cfg.device)
         self.seqs: dict[int, Sequence] = {}
         self._profiler = None
+        self.deferred_output = bool(cfg.deferred_output)
+        self._in_flight: _InFlight | None = None
+        # two pinned buffers take turns: a step's tokens are read while the next step's are on their way
+        self._stages = [_Stage(cfg.max_num_seqs, pinned=torch.device(cfg.device).type == "cuda") for _ in range(2)]
+        self._next_stage = 0
 
     def _cache_budget(self) -> int:
         """Bytes for the cache: the share of device memory ``gpu_memory_utilization`` allows
@@ -113,34 +151,80 @@ class LLMEngine:
         return out
 
     def is_finished(self) -> bool:
-        return self.scheduler.is_finished()
+        return self.scheduler.is_finished() and self._in_flight is None
 
     # ------------------------------------------------------------------ one step
 
     def step(self) -> list[Sequence]:
-        """Runs one scheduled batch; returns the sequences that left in it."""
-        batch = self.scheduler.schedule()
-        done = self.scheduler.take_rejected()
-        if batch is None:
-            return done
+        """Runs one scheduled batch; returns the sequences that left in it.
+
+        With ``deferred_output`` (the default, and the reference's way, atom/model_engine/model_runner.py
+        :358-392) the batch that follows a decode step is launched before the host reads that step's
+        tokens, whenever the scheduler can tell what it will hold (``Scheduler.schedule_ahead``): the
+        new step takes its tokens from the sampler's output on the device.  A request that turns out to
+        have finished is run once too often and that result dropped."""
+        done = []
+        if self._in_flight is None:
+            batch = self.scheduler.schedule()
+            done += self.scheduler.take_rejected()
+            if batch is None:
+                return done
+            self._in_flight = self._launch(batch, None)
+        running = self._in_flight
+        ahead = None
+        if self.deferred_output:
+            batch = self.scheduler.schedule_ahead(running.batch)
+            if batch is not None:
+                ahead = self._launch(batch, {it.seq.id: k for k, it in enumerate(running.finals)})
+        done += self._finish(running)
+        self._in_flight = ahead
+        return done
+
+    def _launch(self, batch, sampled_rows: dict[int, int] | None) -> "_InFlight":
+        """Queues the batch's step and its sampling on the device; waits for nothing."""
         start = time.time()
         with torch.profiler.record_function(self._run_label(batch)):
-            logits = self.core.step(batch.entries())
-        sampled = {}
+            logits = self.core.step(batch.entries(sampled_rows))
         finals = [it for it in batch.items if it.is_final]
+        flight = _InFlight(batch, finals, start)
         if finals:
+            # the tokens stay on the device for a step scheduled ahead and go to pinned memory for the host
             tokens = self.sampler(logits, [it.seq.sampling_params for it in finals],
                                   [it.seq.seed for it in finals],
-                                  [it.seq.num_completion_tokens for it in finals])
-            want_lp = any(it.seq.sampling_params.logprobs for it in finals)
-            lps = self.sampler.logprobs(logits, tokens).tolist() if want_lp else None
-            host = tokens.tolist()
-            for k, it in enumerate(finals):
+                                  [it.seq.num_completion_tokens for it in finals],
+                                  out=self.core.sampled[:len(finals)])
+            stage = self._stages[self._next_stage]
+            self._next_stage = (self._next_stage + 1) % len(self._stages)
+            if len(finals) > stage.tokens.numel():
+                stage.grow(len(finals))
+            flight.tokens = stage.tokens[:len(finals)]
+            flight.tokens.copy_(tokens, non_blocking=True)
+            if any(it.seq.sampling_params.logprobs for it in finals):
+                flight.logprobs = stage.logprobs[:len(finals)]
+                flight.logprobs.copy_(self.sampler.logprobs(logits, tokens), non_blocking=True)
+            flight.ready.record()
+        return flight
+
+    def _finish(self, flight: "_InFlight") -> list[Sequence]:
+        """Waits for the step's tokens and hands them to the scheduler."""
+        sampled = {}
+        if flight.finals:
+            flight.ready.synchronize()
+            host = flight.tokens.tolist()
+            lps = flight.logprobs.tolist() if flight.logprobs is not None else None
+            for k, it in enumerate(flight.finals):
                 sampled[it.seq.id] = host[k]
-                if lps is not None and it.seq.sampling_params.logprobs:
+                if (lps is not None and it.seq.sampling_params.logprobs
+                        and it.seq.status == SequenceStatus.RUNNING):
                     it.seq.logprobs.append(lps[k])
-        done += self.scheduler.postprocess(batch, sampled, time.time() - start)
-        return done
+        return self.scheduler.postprocess(flight.batch, sampled, time.time() - flight.start)
+
+    def drain(self) -> list[Sequence]:
+        """Finishes a step that is still running without starting another."""
+        if self._in_flight is None:
+            return []
+        flight, self._in_flight = self._in_flight, None
+        return self._finish(flight)
 
     @staticmethod
     def _run_label(batch) -> str:
@@ -184,8 +268,9 @@ class LLMEngine:
                     outputs[seq.id] = self._output(seq)
                     del pending[seq.id]
                     self.seqs.pop(seq.id, None)
-            if self.scheduler.is_finished() and pending:
+            if self.is_finished() and pending:
                 raise RuntimeError(f"the scheduler is idle but {len(pending)} request(s) never finished")
+        self.drain()   # a step launched ahead for requests that have all finished
         return [outputs[i] for i in sorted(outputs)]
 
     # ------------------------------------------------------------------ profiling

@@ -54,13 +54,18 @@ class ScheduledBatch:
     def num_prefill(self) -> int:
         return sum(1 for i in self.items if not i.is_decode)
 
-    def entries(self) -> list[StepEntry]:
+    def entries(self, sampled_rows: dict[int, int] | None = None) -> list[StepEntry]:
+        """``sampled_rows``: for a batch scheduled ahead, sequence id -> the row in which the step before
+        this one samples that sequence's token; its entry names that row instead of the token."""
         out = []
         for it in self.items:
             tokens = it.seq.token_ids[it.start:it.start + it.num_tokens]
             want = [it.num_tokens - 1] if it.is_final else []
             reserve = it.seq.num_tokens if not it.is_decode else None
-            out.append(StepEntry(it.seq.id, tokens, want, reserve))
+            feed = None
+            if it.seq.awaits_token and it.start + it.num_tokens == it.seq.num_tokens:
+                feed = sampled_rows[it.seq.id]
+            out.append(StepEntry(it.seq.id, tokens, want, reserve, feed))
         return out
 
 
@@ -264,6 +269,53 @@ class Scheduler:
             self._last_prompt_time = now
         return batch
 
+    # ------------------------------------------------------------------ the step after a running one
+
+    def schedule_ahead(self, running_batch: ScheduledBatch) -> ScheduledBatch | None:
+        """The batch that follows ``running_batch``, made before that batch's tokens are known, so that
+        the device never waits for the host between two decode steps (the reference's deferred output,
+        atom/model_engine/model_runner.py:358-392, scheduler.py:2127-2133).  Only the steady case is taken:
+        every running request is in ``running_batch`` and gets a token from it, nothing can be admitted
+        (now, or because a request reaches its token count in ``running_batch``), and the pools hold
+        the pages of one more token for all of them.  Every request of
+        ``running_batch`` then ends in a placeholder, and those that cannot finish by their token
+        count decode once more.  In every other case this returns None and changes nothing: the caller
+        waits for the running batch and schedules as usual."""
+        if self._rejected or (self.waiting and len(self.running) < self.max_num_seqs):
+            return None
+        if len(running_batch.items) != len(self.running):
+            return None
+        if any(not it.is_final or it.seq.status != SequenceStatus.RUNNING or it.seq.awaits_token
+               for it in running_batch.items):
+            return None
+        mgr = self.manager
+        plan = []
+        need = [0] * len(mgr.groups)
+        for it in running_batch.items:
+            seq = it.seq
+            # with the token that the running batch gives it
+            if seq.num_completion_tokens + 1 >= seq.max_tokens or seq.num_tokens + 1 >= self.max_model_len:
+                if self.waiting:
+                    return None   # its place goes to a waiting request in the very next step
+                continue
+            after = it.start + it.num_tokens
+            for gi, n in enumerate(mgr.pages_missing(seq.id, after, after + 1)):
+                need[gi] += n
+            plan.append((seq, after))
+        if not plan or len(plan) > min(self.max_num_seqs, self.max_num_batched_tokens):
+            return None
+        if any(n > mgr.num_free_pages(gi) for gi, n in enumerate(need)):
+            return None
+        for it in running_batch.items:
+            it.seq.num_cached_tokens = it.start + it.num_tokens
+            it.seq.is_partial_prefill = False
+            it.seq.append_placeholder()
+        batch = ScheduledBatch()
+        for seq, after in plan:
+            mgr.cover(seq.id, after, after + 1)
+            batch.items.append(ScheduledItem(seq, 1, after, True, True))
+        return batch
+
     # ------------------------------------------------------------------ after the step
 
     def _finish_reason(self, seq: Sequence, token: int) -> str | None:
@@ -292,13 +344,20 @@ class Scheduler:
             self._last_prompt_latency = step_seconds
         for it in batch.items:
             seq = it.seq
-            seq.num_cached_tokens = it.start + it.num_tokens
+            if seq.status != SequenceStatus.RUNNING:
+                continue   # it finished while this batch, scheduled ahead, was running: the result is dropped
+            if not seq.awaits_token:
+                seq.num_cached_tokens = it.start + it.num_tokens
             if not it.is_final:
                 seq.is_partial_prefill = True
                 continue
             seq.is_partial_prefill = False
             token = sampled[seq.id]
-            seq.append_token(token)
+            if seq.awaits_token:   # scheduled ahead meanwhile: the placeholder becomes the token
+                seq.resolve_placeholder(token)
+                self.core.resolve(seq.id, seq.num_tokens - 1, token)
+            else:
+                seq.append_token(token)
             if seq.first_token_time == 0.0:
                 seq.first_token_time = now
             reason = self._finish_reason(seq, token)

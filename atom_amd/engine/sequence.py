@@ -28,6 +28,7 @@ class Sequence:
         self.num_prompt_tokens = len(self.token_ids)
         self.num_cached_tokens = 0          # tokens whose keys and values are in the cache
         self.is_partial_prefill = False
+        self.awaits_token = False           # the last token is a placeholder for one still on the device
         self.sampling_params = sp
         self.temperature = sp.temperature
         self.max_tokens = sp.max_tokens
@@ -63,3 +64,20 @@ class Sequence:
 
     def append_token(self, token_id: int) -> None:
         self.token_ids.append(int(token_id))
+
+    # A step may be scheduled before the host has read the token that the step before it sampled (the
+    # reference appends a placeholder and overwrites it, atom/model_engine/scheduler.py:2127-2133,
+    # 2196-2247): the sequence then ends in a placeholder until ``resolve_placeholder``.
+    PLACEHOLDER = 0
+
+    def append_placeholder(self) -> None:
+        if self.awaits_token:
+            raise AssertionError(f"sequence {self.id} already ends in a token that is not known yet")
+        self.token_ids.append(self.PLACEHOLDER)
+        self.awaits_token = True
+
+    def resolve_placeholder(self, token_id: int) -> None:
+        if not self.awaits_token:
+            raise AssertionError(f"sequence {self.id} awaits no token")
+        self.token_ids[-1] = int(token_id)
+        self.awaits_token = False

@@ -110,7 +110,7 @@ class HipKernels:
         except OSError as e:
             raise KernelError(f"could not load the kernel library {path}: {e}") from e
         self.path = path
-        for fn in ("atom_embedding", "atom_rmsnorm", "atom_silu_mul", "atom_qk_norm_rope_kv_write",
+        for fn in ("atom_embedding", "atom_feed_tokens", "atom_rmsnorm", "atom_silu_mul", "atom_qk_norm_rope_kv_write",
                    "atom_gemm_skinny", "atom_gemm_skinny_splits", "atom_gemm_skinny_supports", "atom_splitk_reduce",
                    "atom_paged_attention_generic", "atom_gemm_f32", "atom_sample", "atom_exponential_noise",
                    "atom_attention_mfma_supports", "atom_attention_decode", "atom_attention_prefill",
@@ -230,6 +230,17 @@ class HipKernels:
             _ptr(table), self._code(table), _ptr(ids), _ptr(out), self._code(out), tokens, hidden, vocab,
             self._stream()))
         return out
+
+    def feed_tokens(self, ids: torch.Tensor, source: torch.Tensor, sampled: torch.Tensor) -> torch.Tensor:
+        """``ids[t] = sampled[source[t]]`` where ``source[t] >= 0`` (all int32, in place): token ids that the
+        last step's sampler left on the device."""
+        n = ids.numel()
+        self._check("token ids", ids, torch.int32, (n,))
+        self._check("token sources", source, torch.int32, (n,))
+        self._check("sampled ids", sampled, torch.int32, (None,))
+        self._done("feed_tokens", self.lib.atom_feed_tokens(
+            _ptr(ids), _ptr(source), _ptr(sampled), n, sampled.numel(), self._stream()))
+        return ids
 
     def rmsnorm(self, x, weight, eps: float, out, residual=None, mode: str = "plain", rows=None):
         """mode 'plain': out = norm(x); 'init': residual = x, out = norm(x);

@@ -24,11 +24,12 @@ class Sampler:
         self.device = torch.device(device)
 
     def __call__(self, logits: torch.Tensor, params: list[SamplingParams], seeds: list[int],
-                 counters: list[int]) -> torch.Tensor:
-        """``logits`` float32 [rows, vocab]; returns int32 [rows] on the device."""
+                 counters: list[int], out: torch.Tensor | None = None) -> torch.Tensor:
+        """``logits`` float32 [rows, vocab]; returns int32 [rows] on the device (``out`` if given)."""
         rows = logits.shape[0]
         assert rows == len(params) == len(seeds) == len(counters)
-        out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+        if out is None:
+            out = torch.empty(rows, dtype=torch.int32, device=logits.device)
         temps = np.array([p.temperature if p.temperature > SAMPLER_EPS else 0.0 for p in params], dtype=np.float32)
         if not temps.any():  # all greedy
             self.ops.sample(logits, None, out)

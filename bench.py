@@ -65,6 +65,8 @@ def main() -> int:
                     help="instead: N requests with prompts of 64..3072 tokens through the scheduler, prompt portions of "
                          "512 tokens beside running decodes, 128 output tokens each; prints its own line")
     ap.add_argument("--enforce-eager", action="store_true")
+    ap.add_argument("--no-deferred-output", action="store_true",
+                    help="read every step's tokens before the next step is launched")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not built")
@@ -89,7 +91,8 @@ def main() -> int:
     llm = LLMEngine("qwen3-8b-random", model_config=cfg, load_dummy="random", seed=2, dtype="bf16",
                     max_model_len=max_model_len, kv_cache_block_size=block,
                     num_kvcache_blocks=max_seqs * max_model_len // block, max_num_seqs=max_seqs,
-                    max_num_batched_tokens=16384, enforce_eager=args.enforce_eager)
+                    max_num_batched_tokens=16384, enforce_eager=args.enforce_eager,
+                    deferred_output=not args.no_deferred_output)
     torch.cuda.synchronize()
     print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
     gen = torch.Generator().manual_seed(2)
@@ -193,7 +196,7 @@ def main() -> int:
                    "num_key_value_heads": raw["num_key_value_heads"], "head_dim": raw["head_dim"],
                    "intermediate_size": raw["intermediate_size"], "vocab_size": vocab,
                    "max_model_len": max_model_len, "kv_block_size": block, "decode_steps": steps,
-                   "hip_graphs": not args.enforce_eager},
+                   "hip_graphs": not args.enforce_eager, "deferred_output": not args.no_deferred_output},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": {f"decode_b{b}": round(b * results[b][2] / results[b][0], 2) for b in points if b != args.batch},

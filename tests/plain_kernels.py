@@ -23,6 +23,11 @@ class PlainKernels:
         out.copy_(table[ids.long()].to(out.dtype))
         return out
 
+    def feed_tokens(self, ids, source, sampled):
+        take = source >= 0
+        ids[take] = sampled[source[take].long()]
+        return ids
+
     def rmsnorm(self, x, weight, eps, out, residual=None, mode="plain", rows=None):
         xs = x.to(WIDE)
         if rows is not None:

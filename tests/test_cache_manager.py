@@ -303,3 +303,31 @@ def test_prefix_cache_random_orders():
 def test_prefix_cache_refuses_window_groups():
     with pytest.raises(ValueError):
         CacheManager([GroupSpec(4, 8, window=6)], 2, prefix_caching=True)
+
+
+def test_a_page_is_named_only_when_all_its_tokens_are_known():
+    """A token that ran before the host knew it (read on the device) keeps its page out of the prefix
+    cache until ``amend`` tells its value."""
+    mgr = CacheManager([GroupSpec(4, 8)], 2, prefix_caching=True)
+    mgr.open("a")
+    mgr.cover("a", 0, 7)
+    mgr.commit("a", 7, [1, 2, 3, 4, 5, 6, 7])
+    assert mgr.pools[0].hash_of(mgr.block_table("a", 0)[0]) is not None
+    mgr.cover("a", 7, 8)
+    mgr.commit("a", 8, [0], last_unknown=True)            # fills the second page, value unknown
+    assert mgr.awaited_position("a") == 7
+    assert mgr.pools[0].hash_of(mgr.block_table("a", 0)[1]) is None
+    with pytest.raises(AssertionError):
+        mgr.commit("a", 9, [0], last_unknown=True)         # never two at once
+    with pytest.raises(AssertionError):
+        mgr.amend("a", 6, 9)
+    mgr.amend("a", 7, 8)
+    assert mgr.awaited_position("a") is None
+    assert mgr.pools[0].hash_of(mgr.block_table("a", 0)[1]) is not None
+    mgr.close("a")
+    mgr.open("b")
+    assert mgr.match_prefix("b", [1, 2, 3, 4, 5, 6, 7, 8, 9]) == 8      # found under the amended token
+    mgr.close("b")
+    mgr.open("c")
+    assert mgr.match_prefix("c", [1, 2, 3, 4, 5, 6, 7, 0, 9]) == 4      # not under the placeholder
+    mgr.check()

@@ -79,3 +79,91 @@ def test_step_rejects_bad_input():
     with pytest.raises(ValueError):
         core.step([StepEntry("a", list(range(129)), [])])   # 128 positions
     assert not core.manager.live_requests()
+
+
+# ------------------------------------------------------------------ steps launched before the last one's tokens are read
+
+
+def _engine(deferred, which="B", **kw):
+    from helpers import tiny_folder
+    from tiny import PAGE
+    from atom_amd import LLMEngine
+
+    kw.setdefault("num_kvcache_blocks", 64)
+    kw.setdefault("max_num_seqs", 4)
+    return LLMEngine(tiny_folder(which), dtype="fp32", ops=PlainKernels(), device="cpu",
+                     kv_cache_block_size=PAGE[which], deferred_output=deferred, **kw)
+
+
+def _same(a, b):
+    assert [o["token_ids"] for o in a] == [o["token_ids"] for o in b]
+    assert [o["finish_reason"] for o in a] == [o["finish_reason"] for o in b]
+    for x, y in zip(a, b):
+        assert (x["logprobs"] is None) == (y["logprobs"] is None)
+        if x["logprobs"]:
+            assert x["logprobs"] == pytest.approx(y["logprobs"], abs=1e-5)
+
+
+def _idle(llm):
+    llm.core.manager.check()
+    assert llm.is_finished() and not llm.core.manager.live_requests()
+    assert all(pool.num_free == pool.num_pages for pool in llm.core.manager.pools)
+
+
+def test_steps_launched_ahead_change_no_token():
+    """Greedy, seeded temperature and log-probabilities; requests of different lengths that leave at
+    different times; more requests than run at once; so few pages that requests are preempted."""
+    from atom_amd import SamplingParams
+
+    prompts = [random_ids("B", n, 7 + n) for n in (9, 40, 23, 5, 31, 12)]
+    params = [SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True),
+              SamplingParams(temperature=0.7, max_tokens=20, ignore_eos=True, seed=5),
+              SamplingParams(temperature=0.0, max_tokens=7, ignore_eos=True, logprobs=True),
+              SamplingParams(temperature=1.0, top_k=5, max_tokens=9, ignore_eos=True, seed=2),
+              SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True),
+              SamplingParams(temperature=0.0, max_tokens=15, ignore_eos=True)]
+    for kw in ({}, {"max_num_seqs": 2}, {"num_kvcache_blocks": 12}):
+        plain, ahead = _engine(False, **kw), _engine(True, **kw)
+        _same(plain.generate(prompts, params), ahead.generate(prompts, params))
+        _idle(ahead)
+        if "num_kvcache_blocks" in kw:
+            assert ahead.scheduler.total_preemptions > 0
+        else:
+            assert ahead.core.steps_run == plain.core.steps_run     # counts decide these ends: no step is wasted
+
+
+def test_a_request_that_ends_on_a_token_is_run_once_more_and_that_result_dropped():
+    from atom_amd import SamplingParams
+
+    prompts = [random_ids("B", n, 3 * n) for n in (9, 17, 26)]
+    sp = SamplingParams(temperature=0.0, max_tokens=14, ignore_eos=True)
+    free = _engine(False).generate(prompts, sp)
+    eos = free[1]["token_ids"][4]
+    sp = SamplingParams(temperature=0.0, max_tokens=14)
+    plain, ahead = _engine(False, eos_token_id=eos), _engine(True, eos_token_id=eos)
+    a, b = plain.generate(prompts, sp), ahead.generate(prompts, sp)
+    _same(a, b)
+    assert b[1]["finish_reason"] == "eos" and len(b[1]["token_ids"]) <= 5
+    _idle(ahead)
+    plain, ahead = _engine(False, eos_token_id=eos), _engine(True, eos_token_id=eos)
+    _same(plain.generate(prompts[1:2], sp), ahead.generate(prompts[1:2], sp))
+    assert ahead.core.steps_run == plain.core.steps_run + 1
+    _idle(ahead)
+
+
+def test_pages_filled_by_steps_launched_ahead_are_found_under_their_real_tokens():
+    """The prefix cache names a page only once the token that a step read on the device is known."""
+    from atom_amd import SamplingParams
+
+    prompt = random_ids("B", 13, 1)
+    sp = SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=True)
+    ahead = _engine(True)
+    first = ahead.generate([prompt], sp)[0]["token_ids"]
+    longer = prompt + first + random_ids("B", 6, 2)
+    hits_before = ahead.core.manager.pools[0].hits
+    again = ahead.generate([longer], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))[0]
+    assert ahead.core.manager.pools[0].hits - hits_before == (len(prompt) + len(first) - 1) // 8
+    fresh = _engine(False, enable_prefix_caching=False).generate(
+        [longer], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))[0]
+    assert again["token_ids"] == fresh["token_ids"]
+    _idle(ahead)

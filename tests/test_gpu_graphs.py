@@ -81,3 +81,38 @@ def test_stateful_mixer_is_not_graphed():
         assert not DecodeGraphs(core, [1, 2], 128).usable
     finally:
         del core.model.blocks[0].mixer.graph_safe
+
+
+@pytest.mark.parametrize("graph_sizes", [None, [4]])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tokens_read_on_the_device(dtype, graph_sizes):
+    """A step whose entries name rows of the sampler's output instead of tokens gives the logits of the
+    step that is handed the same tokens by the host; rows are taken in any order, and a step may mix both."""
+    which = "B"
+    prompts = {f"f{k}": random_ids(which, n, 70 + k) for k, n in enumerate([20, 9, 33])}
+    nxt = {"f0": 5, "f1": 300, "f2": 17}
+
+    def run(fed: dict):
+        core = make_core(which, dtype, gpu_ops(), "cuda:0", num_pages=32, page_size=8, graph_sizes=graph_sizes)
+        for rid, ids in prompts.items():
+            core.step([StepEntry(rid, ids, [])])
+        core.sampled[:4] = torch.tensor([nxt["f2"], 0, nxt["f0"], nxt["f1"]], dtype=torch.int32, device="cuda:0")
+        rows = {"f2": 0, "f0": 2, "f1": 3}
+        entries = [StepEntry(rid, [0] if rid in fed else [nxt[rid]], [0], None, rows[rid] if rid in fed else None)
+                   for rid in prompts]
+        out = core.step(entries).cpu()
+        if graph_sizes:
+            assert core.graphs.replays == 1
+        return out
+
+    given = run({})
+    assert torch.equal(run({"f0", "f1", "f2"}), given)
+    assert torch.equal(run({"f1"}), given)
+    # and beside a prompt portion, where the step is not a graph's
+    core = make_core(which, dtype, gpu_ops(), "cuda:0", num_pages=32, page_size=8, graph_sizes=graph_sizes)
+    core.step([StepEntry("f0", prompts["f0"], [])])
+    core.sampled[1] = nxt["f0"]
+    mixed = core.step([StepEntry("f0", [0], [0], None, 1), StepEntry("f2", prompts["f2"], [])])
+    torch.testing.assert_close(mixed.cpu()[0], given[0], rtol=0, atol=(1e-4 if dtype == "float32" else 3e-2) * float(given.abs().max()))
+    with pytest.raises(ValueError):
+        core.step([StepEntry("f0", [0, 0], [0], None, 1)])

@@ -572,3 +572,15 @@ def test_deferred_sum_readers():
         outs.append((q, kc, vc))
     for a, b in zip(*outs):
         close(a, b.double(), torch.bfloat16, scale=float(b.abs().max()) * 2)
+
+
+def test_feed_tokens():
+    ops = gpu_ops()
+    gen = torch.Generator().manual_seed(3)
+    for n in (1, 7, 300):
+        ids = torch.randint(0, 1000, (n,), generator=gen, dtype=torch.int32)
+        sampled = torch.randint(1000, 2000, (9,), generator=gen, dtype=torch.int32)
+        source = torch.randint(-1, 9, (n,), generator=gen, dtype=torch.int32)
+        want = torch.where(source >= 0, sampled[source.clamp(min=0).long()], ids)
+        got = ops.feed_tokens(ids.cuda(), source.cuda(), sampled.cuda())
+        assert torch.equal(got.cpu(), want)

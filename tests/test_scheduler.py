@@ -30,6 +30,10 @@ class FakeCore:
         if rid in self.manager:
             self.manager.close(rid)
 
+    def resolve(self, rid, position, token):
+        if rid in self.manager and self.manager.awaited_position(rid) == position:
+            self.manager.amend(rid, position, token)
+
 
 def make(blocks=100, block=4, window_group=None, prefix_caching=False, **kw):
     raw = {**TINY_C, "max_position_embeddings": 4096, "eos_token_id": 2}
@@ -324,3 +328,100 @@ def test_preempted_request_finds_its_own_pages_again():
     batch = sched.schedule()
     item = [it for it in batch.items if it.seq is b][0]
     assert item.start >= 8, "the pages it filled before it was preempted are found by their content"
+
+
+# ------------------------------------------------------------------ the step after a running one
+
+
+def _decoding(sched, lengths, **sp):
+    """Requests of these prompt lengths, prefilled and one token in."""
+    seqs = [seq(range(10 * k, 10 * k + n), **sp) for k, n in enumerate(lengths)]
+    for s in seqs:
+        sched.add(s)
+    run(sched, sched.schedule())
+    return seqs
+
+
+def test_schedule_ahead_takes_the_steady_decode_case():
+    sched, core = make(blocks=40, block=4)
+    a, b = _decoding(sched, [6, 9], max_tokens=8, ignore_eos=True)
+    running = sched.schedule()
+    assert [it.is_decode for it in running.items] == [True, True]
+    ahead = sched.schedule_ahead(running)
+    assert [(it.seq.id, it.start, it.num_tokens) for it in ahead.items] == [(a.id, 7, 1), (b.id, 10, 1)]
+    assert a.awaits_token and b.awaits_token and a.num_tokens == 8 and a.num_cached_tokens == 7
+    entries = ahead.entries({a.id: 0, b.id: 1})
+    assert [(e.tokens, e.feed) for e in entries] == [([Sequence.PLACEHOLDER], 0), ([Sequence.PLACEHOLDER], 1)]
+    # the running batch's tokens arrive: the placeholders become them, nothing else moves
+    sched.postprocess(running, {a.id: 31, b.id: 32})
+    assert a.token_ids[-1] == 31 and b.token_ids[-1] == 32 and not a.awaits_token
+    assert a.num_tokens == 8 and a.num_cached_tokens == 7 and a.num_completion_tokens == 2
+    sched.postprocess(ahead, {a.id: 41, b.id: 42})
+    assert a.token_ids[-2:] == [31, 41] and a.num_cached_tokens == 8
+    core.manager.check()
+
+
+def test_schedule_ahead_leaves_out_what_finishes_by_its_count_and_drops_what_finished_meanwhile():
+    sched, core = make(blocks=40, block=4)
+    a, b, c = _decoding(sched, [5, 6, 7], max_tokens=9)
+    a.max_tokens = 3                       # one token in; the running batch gives the second, the next the third
+    running = sched.schedule()
+    ahead = sched.schedule_ahead(running)
+    assert [it.seq.id for it in ahead.items] == [a.id, b.id, c.id]
+    done = sched.postprocess(running, {a.id: 9, b.id: 2, c.id: 9})      # b samples eos (2)
+    assert [s.id for s in done] == [b.id] and b.leave_reason == "eos" and b.id not in core.manager
+    running2 = ahead
+    ahead2 = sched.schedule_ahead(running2)
+    assert ahead2 is None                  # b is in the running batch but runs no more: not the steady case
+    done = sched.postprocess(running2, {a.id: 9, b.id: 77, c.id: 9})
+    assert [s.id for s in done] == [a.id] and a.leave_reason == "max_tokens"
+    assert b.token_ids[-1] == 2 and b.num_completion_tokens == 2          # the token sampled for b after eos is dropped
+    batch = sched.schedule()
+    assert [it.seq.id for it in batch.items] == [c.id]
+    assert sched.schedule_ahead(batch) is not None
+    core.manager.check()
+
+
+def test_schedule_ahead_skips_a_request_at_its_last_token():
+    sched, core = make(blocks=40, block=4)
+    a, b = _decoding(sched, [5, 6], max_tokens=5, ignore_eos=True)
+    a.max_tokens = 2
+    running = sched.schedule()
+    ahead = sched.schedule_ahead(running)
+    assert [it.seq.id for it in ahead.items] == [b.id] and a.awaits_token
+    done = sched.postprocess(running, {a.id: 7, b.id: 8})
+    assert [s.id for s in done] == [a.id] and a.token_ids[-1] == 7 and a.leave_reason == "max_tokens"
+    core.manager.check()
+
+
+def test_schedule_ahead_declines_and_changes_nothing():
+    # a request waits and could be admitted
+    sched, core = make(blocks=40, block=4)
+    a, = _decoding(sched, [6], max_tokens=9)
+    running = sched.schedule()
+    sched.add(seq(range(50, 55)))                   # arrives while the batch runs
+    assert sched.schedule_ahead(running) is None and not a.awaits_token
+    # a prompt that ends in the running batch decodes in the next: its first token too is read on the device
+    sched.postprocess(running, {a.id: 5})
+    running = sched.schedule()
+    assert [it.is_decode for it in running.items] == [True, False]
+    ahead = sched.schedule_ahead(running)
+    assert [(it.start, it.is_decode) for it in ahead.items] == [(8, True), (5, True)]
+    # ... but a full house keeps the waiting request out, so decoding runs ahead
+    sched, core = make(blocks=40, block=4, max_num_seqs=2)
+    a, b = _decoding(sched, [6, 7], max_tokens=9)
+    sched.add(seq(range(50, 55)))
+    running = sched.schedule()
+    assert sched.schedule_ahead(running) is not None
+    # no page for the next token: left to the ordinary path, which preempts
+    sched, core = make(blocks=4, block=4)
+    a, b = _decoding(sched, [7, 7], max_tokens=9, ignore_eos=True)
+    running = sched.schedule()                      # positions 7: the last slots of the second pages
+    before = (a.num_tokens, a.num_cached_tokens, core.manager.num_free_pages(0))
+    assert sched.schedule_ahead(running) is None
+    assert (a.num_tokens, a.num_cached_tokens, core.manager.num_free_pages(0)) == before and not a.awaits_token
+    # an unfinished prompt in the running batch
+    sched, core = make(blocks=100, block=4, max_num_batched_tokens=64)
+    sched.add(seq(range(100)))
+    running = sched.schedule()
+    assert not running.items[0].is_final and sched.schedule_ahead(running) is None
