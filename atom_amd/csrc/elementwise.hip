@@ -6,18 +6,116 @@
 // the residual stream and norm weights are always float32.
 #include "common.h"
 
+// Eight consecutive elements, moved with 16- and 32-byte accesses.
+template <typename T>
+struct Vec8;
+template <>
+struct Vec8<float> {
+  float4 a, b;
+  __device__ __forceinline__ void get(float* f) const {
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+  }
+  __device__ __forceinline__ void set(const float* f) {
+    a = make_float4(f[0], f[1], f[2], f[3]);
+    b = make_float4(f[4], f[5], f[6], f[7]);
+  }
+};
+template <>
+struct Vec8<bf16_t> {
+  __attribute__((ext_vector_type(8))) __bf16 v;
+  __device__ __forceinline__ void get(float* f) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = static_cast<float>(v[i]);
+  }
+  __device__ __forceinline__ void set(const float* f) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = static_cast<bf16_t>(f[i]);
+  }
+};
+
 // An input that is still a sum: `splits` float32 slices [rows, width] `stride` elements apart, as the
 // skinny matrix product leaves them when it cuts K, plus an optional bias over the width.  Readers
 // add the slices in slice order.  `partial == nullptr`: the input is an ordinary tensor.
+//
+// The readers below issue the loads of several slices (and several elements) before they use any of
+// them: a kernel that reads a sum waits for memory once per group of slices, not once per slice.  A
+// group is filled up by reading the last slice again (a cache hit) instead of branching.
 struct SplitSum {
   const float* partial;
   const float* bias;
   size_t stride;
   int splits;
+
+  // the elements at offset[0..N-1] (bias columns col[0..N-1]); kGroup: slices whose loads are in flight together
+  template <int N, int kGroup = 4>
+  __device__ __forceinline__ void at_many(const size_t (&offset)[N], const int (&col)[N], float (&out)[N]) const {
+#pragma unroll
+    for (int n = 0; n < N; ++n) out[n] = 0.f;
+    for (int s0 = 0; s0 < splits; s0 += kGroup) {
+      float part[N][kGroup];
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        const float* slice = partial + (size_t)min(s0 + u, splits - 1) * stride;
+#pragma unroll
+        for (int n = 0; n < N; ++n) part[n][u] = slice[offset[n]];
+      }
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        const bool live = s0 + u < splits;
+#pragma unroll
+        for (int n = 0; n < N; ++n) out[n] += live ? part[n][u] : 0.f;
+      }
+    }
+    if (bias) {
+#pragma unroll
+      for (int n = 0; n < N; ++n) out[n] += bias[col[n]];
+    }
+  }
+
   __device__ __forceinline__ float at(size_t offset, int col) const {
-    float v = 0.f;
-    for (int s = 0; s < splits; ++s) v += partial[(size_t)s * stride + offset];
-    return bias ? v + bias[col] : v;
+    const size_t offsets[1] = {offset};
+    const int cols[1] = {col};
+    float out[1];
+    at_many<1>(offsets, cols, out);
+    return out[0];
+  }
+
+  // N runs of eight consecutive elements, each at a 32-byte aligned offset (bias columns col[n] ..)
+  template <int N, int kGroup = 4>
+  __device__ __forceinline__ void runs_of_8(const size_t (&offset)[N], const int (&col)[N], float (&out)[N][8]) const {
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[n][e] = 0.f;
+    for (int s0 = 0; s0 < splits; s0 += kGroup) {
+      Vec8<float> part[N][kGroup];
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        const float* slice = partial + (size_t)min(s0 + u, splits - 1) * stride;
+#pragma unroll
+        for (int n = 0; n < N; ++n) part[n][u] = *reinterpret_cast<const Vec8<float>*>(slice + offset[n]);
+      }
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        const bool live = s0 + u < splits;
+#pragma unroll
+        for (int n = 0; n < N; ++n) {
+          float v[8];
+          part[n][u].get(v);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) out[n][e] += live ? v[e] : 0.f;
+        }
+      }
+    }
+    if (bias) {
+#pragma unroll
+      for (int n = 0; n < N; ++n) {
+        float v[8];
+        reinterpret_cast<const Vec8<float>*>(bias + col[n])->get(v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[n][e] += v[e];
+      }
+    }
   }
 };
 
@@ -116,32 +214,6 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, float* __restrict__ resi
 // The same for widths that are a multiple of 8: a thread keeps VPT groups of 8 consecutive
 // elements in registers, all loads of a row are issued at once (16- and 32-byte accesses) and
 // nothing goes through LDS but the reduction.  blockDim.x * 8 * VPT >= width.
-template <typename T>
-struct Vec8;
-template <>
-struct Vec8<float> {
-  float4 a, b;
-  __device__ __forceinline__ void get(float* f) const {
-    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
-  }
-  __device__ __forceinline__ void set(const float* f) {
-    a = make_float4(f[0], f[1], f[2], f[3]);
-    b = make_float4(f[4], f[5], f[6], f[7]);
-  }
-};
-template <>
-struct Vec8<bf16_t> {
-  __attribute__((ext_vector_type(8))) __bf16 v;
-  __device__ __forceinline__ void get(float* f) const {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = static_cast<float>(v[i]);
-  }
-  __device__ __forceinline__ void set(const float* f) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = static_cast<bf16_t>(f[i]);
-  }
-};
-
 template <typename T, int VPT>
 __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, float* __restrict__ residual,
                                    const float* __restrict__ weight, T* __restrict__ y,
@@ -163,29 +235,22 @@ __global__ void rmsnorm_vec_kernel(const T* __restrict__ x, float* __restrict__ 
       if (mode == 2) rv[j] = *reinterpret_cast<const Vec8<float>*>(rr + i);
     }
   }
+  if (xsum.partial) {
+    // groups beyond the width read the row's last group again and are not used
+    size_t offsets[VPT];
+    int cols[VPT];
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+      cols[j] = min((int)(threadIdx.x + j * blockDim.x) * 8, width - 8);
+      offsets[j] = (size_t)src * width + cols[j];
+    }
+    xsum.runs_of_8<VPT, (VPT == 1 ? 8 : 4)>(offsets, cols, vals);
+  }
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int i = (threadIdx.x + j * blockDim.x) * 8;
     if (i < width) {
-      if (xsum.partial) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) vals[j][e] = 0.f;
-        const float* base = xsum.partial + (size_t)src * width + i;
-        for (int sp = 0; sp < xsum.splits; ++sp) {
-          float part[8];
-          reinterpret_cast<const Vec8<float>*>(base + (size_t)sp * xsum.stride)->get(part);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) vals[j][e] += part[e];
-        }
-        if (xsum.bias) {
-          float part[8];
-          reinterpret_cast<const Vec8<float>*>(xsum.bias + i)->get(part);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) vals[j][e] += part[e];
-        }
-      } else {
-        xv[j].get(vals[j]);
-      }
+      if (!xsum.partial) xv[j].get(vals[j]);
       if (mode == 2) {
         float add[8];
         rv[j].get(add);
@@ -265,9 +330,18 @@ __global__ void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ y, int 
   if (idx >= total) return;
   const size_t row = idx / inter;
   const int col = (int)(idx - row * inter);
-  const float g = xsum.partial ? xsum.at(row * 2 * inter + col, col) : to_f32(x[row * 2 * inter + col]);
-  const float u = xsum.partial ? xsum.at(row * 2 * inter + inter + col, inter + col)
-                               : to_f32(x[row * 2 * inter + inter + col]);
+  float g, u;
+  if (xsum.partial) {
+    const size_t offsets[2] = {row * 2 * inter + col, row * 2 * inter + inter + col};
+    const int cols[2] = {col, inter + col};
+    float both[2];
+    xsum.at_many<2>(offsets, cols, both);
+    g = both[0];
+    u = both[1];
+  } else {
+    g = to_f32(x[row * 2 * inter + col]);
+    u = to_f32(x[row * 2 * inter + inter + col]);
+  }
   y[idx] = from_f32<T>(g / (1.f + expf(-g)) * u);
 }
 
@@ -282,25 +356,14 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ x, T* __restrict__ y, 
   const int col = (int)(idx - row * per_row) * 8;
   float g[8], u[8], o[8];
   if (xsum.partial) {
+    const size_t offsets[2] = {row * 2 * inter + col, row * 2 * inter + inter + col};
+    const int cols[2] = {col, inter + col};
+    float both[2][8];
+    xsum.runs_of_8<2>(offsets, cols, both);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) g[e] = u[e] = 0.f;
-    const float* base = xsum.partial + row * 2 * inter + col;
-    for (int sp = 0; sp < xsum.splits; ++sp) {
-      float a[8], b[8];
-      reinterpret_cast<const Vec8<float>*>(base + (size_t)sp * xsum.stride)->get(a);
-      reinterpret_cast<const Vec8<float>*>(base + (size_t)sp * xsum.stride + inter)->get(b);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        g[e] += a[e];
-        u[e] += b[e];
-      }
-    }
-    if (xsum.bias) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        g[e] += xsum.bias[col + e];
-        u[e] += xsum.bias[inter + col + e];
-      }
+    for (int e = 0; e < 8; ++e) {
+      g[e] = both[0][e];
+      u[e] = both[1][e];
     }
   } else {
     const Vec8<T> gv = *reinterpret_cast<const Vec8<T>*>(x + row * 2 * inter + col);
@@ -366,10 +429,7 @@ __global__ void qk_norm_rope_kv_write_kernel(
   const int head = blockIdx.y + head_begin;  // 0..hq-1 q, then hkv k heads, then hkv v heads
   const int lane = threadIdx.x;
   const int row_width = (hq + 2 * hkv) * d;
-  const T* src = qkv + (size_t)t * row_width + (size_t)head * d;
   const size_t src_off = (size_t)t * row_width + (size_t)head * d;
-  // element i of this head's input: the tensor, or the sum of its slices
-  auto in = [&](int i) -> float { return xsum.partial ? xsum.at(src_off + i, head * d + i) : to_f32(src[i]); };
   const bool is_q = head < hq;
   const bool is_k = !is_q && head < hq + hkv;
   const int kv_head = is_q ? 0 : (is_k ? head - hq : head - hq - hkv);
@@ -412,9 +472,36 @@ __global__ void qk_norm_rope_kv_write_kernel(
   const int page = slot / page_size;
   const int off = slot - page * page_size;
 
+  // The head's d values, read once: where the input is a sum of slices, the loads of four elements and
+  // of four slices are in flight together.  They are kept in LDS (the block is this one wave).
+  extern __shared__ float head_vals[];   // d floats
+  for (int i0 = 0; i0 < d; i0 += 4 * kWave) {
+    size_t offsets[4];
+    int cols[4];
+    float got[4];
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const int i = min(i0 + n * kWave + lane, d - 1);   // beyond the head: its last element again, not used
+      offsets[n] = src_off + i;
+      cols[n] = head * d + i;
+    }
+    if (xsum.partial) {
+      xsum.at_many<4>(offsets, cols, got);
+    } else {
+#pragma unroll
+      for (int n = 0; n < 4; ++n) got[n] = to_f32(qkv[offsets[n]]);
+    }
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const int i = i0 + n * kWave + lane;
+      if (i < d) head_vals[i] = got[n];
+    }
+  }
+  __syncthreads();
+
   if (!is_q && !is_k) {  // value head: plain scatter into the transposed page
     T* dst = v_cache + ((size_t)page * hkv + kv_head) * (size_t)d * page_size + off;
-    for (int i = lane; i < d; i += kWave) dst[(size_t)i * page_size] = from_f32<T>(in(i));
+    for (int i = lane; i < d; i += kWave) dst[(size_t)i * page_size] = from_f32<T>(head_vals[i]);
     return;
   }
 
@@ -423,7 +510,7 @@ __global__ void qk_norm_rope_kv_write_kernel(
   if (weight) {
     float ss = 0.f;
     for (int i = lane; i < d; i += kWave) {
-      const float v = in(i);
+      const float v = head_vals[i];
       ss += v * v;
     }
     ss = wave_sum(ss);
@@ -436,8 +523,8 @@ __global__ void qk_norm_rope_kv_write_kernel(
   const float* cs = cos_table + (size_t)pos * half;
   const float* sn = sin_table + (size_t)pos * half;
   for (int j = lane; j < half; j += kWave) {
-    float x1 = in(j);
-    float x2 = in(j + half);
+    float x1 = head_vals[j];
+    float x2 = head_vals[j + half];
     if (weight) {
       x1 = x1 * inv * weight[j];
       x2 = x2 * inv * weight[j + half];
@@ -447,7 +534,7 @@ __global__ void qk_norm_rope_kv_write_kernel(
     dst[j + half] = from_f32<T>(x2 * c + x1 * s);
   }
   for (int i = rotary_dim + lane; i < d; i += kWave) {  // the part that is not rotated
-    float v = in(i);
+    float v = head_vals[i];
     if (weight) v = v * inv * weight[i];
     dst[i] = from_f32<T>(v);
   }
@@ -551,7 +638,8 @@ ATOM_EXPORT int atom_qk_norm_rope_kv_write(
     head_begin = hq + hkv;
   }
   dim3 grid(tokens, hq + 2 * hkv - head_begin), block(kWave);
-  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<T>), grid, block, 0, stream,
+  if ((size_t)d * 4 > 64 * 1024) return ATOM_TOO_LARGE;   // a head's values are kept in LDS
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<T>), grid, block, (size_t)d * 4, stream,
                                                  (const T*)qkv, (T*)q_out, (T*)k_cache, (T*)v_cache, q_weight,
                                                  k_weight, cos_table, sin_table, positions, slots, hq, hkv, d,
                                                  rotary_dim, page_size, eps, write_kv, xsum, head_begin));
