@@ -47,6 +47,10 @@ struct AttnParams {
 
 __device__ __forceinline__ s16x4 as_s16x4(bf16x4 v) { return __builtin_bit_cast(s16x4, v); }
 
+// 2^x for x <= 0 (and -inf): the bare instruction.  Results below the smallest normal number become 0,
+// which a probability may.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 template <int D, int RT, bool DECODE>
 __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
   constexpr bool KX32 = (D % 32 == 0);
@@ -379,13 +383,13 @@ static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
 //
 // Needs D % 64 == 0 and page_size % 8 == 0.
 template <int D, int GH, int TK>
-__global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams p) {
+__global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_tiled_kernel(AttnParams p) {
   constexpr int KCH = D / 32;
   constexpr int DT = D / 16;
   constexpr int RT = 2;
   constexpr int KB = TK / 16;            // blocks of 16 keys in a tile
   constexpr int KSTR = D + 8;            // LDS row of a key, in elements: rows start 4 banks apart
-  constexpr int VSTR = TK + 4;           // LDS row of V^T (one d), in elements
+  constexpr int VSTR = TK + 8;           // LDS row of V^T (one d), in elements: 16-byte aligned, rows 4 banks apart
   constexpr int PT = D * TK / 8 / 256;   // 16-byte pieces of each tile that a thread moves
   __shared__ __attribute__((aligned(16))) bf16_t ks[TK * KSTR];
   __shared__ __attribute__((aligned(16))) bf16_t vs[D * VSTR];
@@ -399,13 +403,24 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
 
   // A block takes two tiles, one after the other: the host lists tiles with the most keys first, so tile b and
   // tile n - 1 - b together are about the same work for every b, and all blocks finish together.
+  constexpr bool TWO = D <= 128;
   for (int pass = 0; pass < 2; ++pass) {
-  const int tile = pass == 0 ? (int)blockIdx.x : p.num_tiles - 1 - (int)blockIdx.x;
-  if (pass == 1 && tile <= (int)blockIdx.x) break;
+  int tile, ygroup;
+  if (TWO) {
+    if (pass == 1) break;
+    const int total = gridDim.x, half = (total + 1) / 2, groups = p.hq / GH;
+    const int item = (int)blockIdx.x < half ? (int)blockIdx.x : total - 1 - ((int)blockIdx.x - half);
+    tile = item / groups;
+    ygroup = item - tile * groups;
+  } else {
+    tile = pass == 0 ? (int)blockIdx.x : p.num_tiles - 1 - (int)blockIdx.x;
+    if (pass == 1 && tile <= (int)blockIdx.x) break;
+    ygroup = blockIdx.y;
+  }
   const int seq = p.tiles[2 * tile];
   const int row_start = p.tiles[2 * tile + 1];
-  const int head = blockIdx.y * GH + (wave % GH);
-  const int kvh = (blockIdx.y * GH) / group;
+  const int head = ygroup * GH + (wave % GH);
+  const int kvh = (ygroup * GH) / group;
   const int sub = wave / GH;
   const int ctx = p.ctx_lens[seq];
   const int q_begin = p.cu_q[seq];
@@ -472,12 +487,17 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
     for (int j = 0; j < PT; ++j) {
       const int q = tid + 256 * j;
       *reinterpret_cast<bf16x8*>(ks + (q / (D / 8)) * KSTR + (q % (D / 8)) * 8) = kreg[j];
-      // a row of V^T is 8-byte aligned only
+      // Within every 32 keys of a V^T row the keys are laid in the order in which the second product
+      // takes them: lane group g holds keys 4 g .. 4 g + 3 and 16 + 4 g .. 16 + 4 g + 3 (what the first
+      // product left it), so these eight lie together at 8 g: key c goes to 8 ((c % 16) / 4) + 4 (c / 16) + c % 4.
       const bf16x4 lo = {vreg[j][0], vreg[j][1], vreg[j][2], vreg[j][3]};
       const bf16x4 hi = {vreg[j][4], vreg[j][5], vreg[j][6], vreg[j][7]};
-      bf16_t* dst = vs + (q / (TK / 8)) * VSTR + (q % (TK / 8)) * 8;
-      *reinterpret_cast<bf16x4*>(dst) = lo;
-      *reinterpret_cast<bf16x4*>(dst + 4) = hi;
+      const int c0 = (q % (TK / 8)) * 8;              // first key of the piece within the tile
+      const int in32 = c0 % 32;
+      const int at_lo = 8 * ((in32 % 16) / 4) + 4 * (in32 / 16);
+      bf16_t* dst = vs + (q / (TK / 8)) * VSTR + (c0 - in32);
+      *reinterpret_cast<bf16x4*>(dst + at_lo) = lo;
+      *reinterpret_cast<bf16x4*>(dst + at_lo + 8) = hi;   // keys c0 + 4 ..: the next lane group
     }
   };
 
@@ -505,35 +525,48 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
           s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q32[rt][j], s[rt][b], 0, 0, 0);
       }
 
-    // ---- softmax update; lane holds keys k0 + 16 b + 4 g + i of row r16
+    // ---- softmax update; lane holds keys k0 + 16 b + 4 g + i of row r16.  The maximum is taken over the
+    //      raw scores and the scale goes into the exponent's multiply-add.  A tile that every row of the
+    //      wave sees whole (all but the last one or two of a causal prompt) needs no masking.
     bf16x8 pb[RT][KB / 2];
     float alpha[RT];
     bool rescale = false;
+    const bool whole = k0 + TK - 1 <= min(pos0, ke - 1) && (p.window <= 0 || k0 >= pos0 + nrows - p.window);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       float sc[4 * KB];
       float mx = -INFINITY;
-      const int hi = min(row_pos[rt], ke - 1);
-      const int lo = p.window > 0 ? row_pos[rt] - p.window + 1 : 0;
+      if (whole) {
 #pragma unroll
-      for (int b = 0; b < KB; ++b)
+        for (int b = 0; b < KB; ++b)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = k0 + 16 * b + 4 * g + i;
-          const bool vis = key <= hi && key >= lo;
-          sc[4 * b + i] = vis ? s[rt][b][i] * p.scale_log2 : -INFINITY;
-          mx = fmaxf(mx, sc[4 * b + i]);
-        }
+          for (int i = 0; i < 4; ++i) {
+            sc[4 * b + i] = s[rt][b][i];
+            mx = fmaxf(mx, sc[4 * b + i]);
+          }
+      } else {
+        const int hi = min(row_pos[rt], ke - 1);
+        const int lo = p.window > 0 ? row_pos[rt] - p.window + 1 : 0;
+#pragma unroll
+        for (int b = 0; b < KB; ++b)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = k0 + 16 * b + 4 * g + i;
+            const bool vis = key <= hi && key >= lo;
+            sc[4 * b + i] = vis ? s[rt][b][i] : -INFINITY;
+            mx = fmaxf(mx, sc[4 * b + i]);
+          }
+      }
       mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
       mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-      const float new_max = fmaxf(run_max[rt], mx);
+      const float new_max = fmaxf(run_max[rt], mx * p.scale_log2);
       const float base = new_max == -INFINITY ? 0.f : new_max;
-      alpha[rt] = exp2f(run_max[rt] - base);
+      alpha[rt] = fast_exp2(run_max[rt] - base);
       rescale = rescale || alpha[rt] != 1.f;
       float psum = 0.f;
 #pragma unroll
       for (int e = 0; e < 4 * KB; ++e) {
-        const float pv = exp2f(sc[e] - base);
+        const float pv = fast_exp2(fmaf(sc[e], p.scale_log2, -base));
         psum += pv;
         pb[rt][e / 8][e % 8] = static_cast<bf16_t>(pv);
       }
@@ -556,10 +589,7 @@ __global__ void __launch_bounds__(256) attention_prefill_tiled_kernel(AttnParams
     for (int h = 0; h < KB / 2; ++h)
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
-        const bf16_t* vrow = vs + (16 * t + r16) * VSTR + 32 * h + 4 * g;
-        const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vrow);
-        const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vrow + 16);
-        const bf16x8 a = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(vs + (16 * t + r16) * VSTR + 32 * h + 8 * g);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
           acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[rt][h], acc[rt][t], 0, 0, 0);
@@ -601,6 +631,7 @@ static int launch_prefill_tiled(const AttnParams& p, int num_tiles, int rows_per
   const int gh = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
   if (rows_per_tile != 32 * (4 / gh)) return ATOM_BAD_SHAPE;
   dim3 grid((num_tiles + 1) / 2, p.hq / gh), block(256);
+  if (D <= 128) grid = dim3(num_tiles * (p.hq / gh), 1);
   constexpr int TK = D <= 128 ? 64 : 32;
   if (gh == 4) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 4, TK>), grid, block, 0, stream, p);
   else if (gh == 2) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 2, TK>), grid, block, 0, stream, p);
