@@ -373,7 +373,7 @@ static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
 //
 // A block of four waves owns a tile of query tokens of GH query heads that share a KV head
 // (GH = 4, 2 or 1, a divisor of the group size): wave w has head (w % GH) and the 32 tokens
-// number (w / GH) of the tile, so a block covers 32 * 4 / GH tokens.  Keys are walked TK (32) at a
+// number (w / GH) of the tile, so a block covers 32 * 4 / GH tokens.  Keys are walked TK (64 or 32) at a
 // time; the block loads each K tile (TK keys x D) and V^T tile (D x TK keys) once, through
 // registers (the next tile's loads are in flight while this one is multiplied) into LDS, where all
 // four waves read them as matrix-core operands.  Products, softmax and layouts are those of the
@@ -401,8 +401,12 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
   const int group = p.hq / p.hkv;
   const int ps = p.page_size;
 
-  // A block takes two tiles, one after the other: the host lists tiles with the most keys first, so tile b and
-  // tile n - 1 - b together are about the same work for every b, and all blocks finish together.
+  // The host lists tiles with the most keys first, so tile b and tile n - 1 - b together are about the same
+  // work for every b.  Head sizes up to 128 fit two blocks on a CU (256 registers a lane): every block takes
+  // one (tile, head group), the grid is one-dimensional, and its first half walks the list from the longest
+  // item down while its second half walks it from the shortest up, so that the two blocks that meet on a
+  // CU (block b and block b + n / 2, as blocks are handed out in order) are a long and a short one.
+  // Larger heads run one block a CU, which takes tile b and then tile n - 1 - b.
   constexpr bool TWO = D <= 128;
   for (int pass = 0; pass < 2; ++pass) {
   int tile, ygroup;
