@@ -250,12 +250,12 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
       mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
       const float new_max = fmaxf(run_max[rt], mx);
       const float base = new_max == -INFINITY ? 0.f : new_max;
-      const float alpha = exp2f(run_max[rt] - base);   // 0 while nothing was seen yet
+      const float alpha = fast_exp2(run_max[rt] - base);   // 0 while nothing was seen yet
       float psum = 0.f;
       bf16x4 pb;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float pv = exp2f(sc[i] - base);
+        const float pv = fast_exp2(sc[i] - base);
         psum += pv;
         pb[i] = static_cast<bf16_t>(pv);
       }
