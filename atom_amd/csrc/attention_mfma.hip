@@ -232,30 +232,43 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
 #pragma unroll
     for (int t = 0; t < DT; ++t) vreg[t] = cur.v[t];
 
-    // ---- softmax update per row tile; lane holds keys k0 + 4g + i of row r16
+    // ---- softmax update per row tile; lane holds keys k0 + 4g + i of row r16.  The maximum is taken over
+    //      the raw scores and the scale goes into the exponent's multiply-add; a block of keys that every
+    //      row sees whole (all but the last of a decode row's) is not masked.
+    const int first_pos = pos0;                                 // the smallest position among the rows
+    const int last_pos = DECODE ? pos0 : pos0 + nrows - 1;
+    const bool whole = k0 + 15 <= min(first_pos, ke - 1) && (p.window <= 0 || k0 >= last_pos - p.window + 1);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       float sc[4];
       float mx = -INFINITY;
-      const int hi = min(row_pos[rt], ke - 1);                        // last visible key
-      const int lo = p.window > 0 ? row_pos[rt] - p.window + 1 : 0;   // first visible key
+      if (whole) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = k0 + 4 * g + i;
-        const bool vis = key <= hi && key >= lo && key >= kb;
-        sc[i] = vis ? s[rt][i] * p.scale_log2 : -INFINITY;
-        mx = fmaxf(mx, sc[i]);
+        for (int i = 0; i < 4; ++i) {
+          sc[i] = s[rt][i];
+          mx = fmaxf(mx, sc[i]);
+        }
+      } else {
+        const int hi = min(row_pos[rt], ke - 1);                        // last visible key
+        const int lo = p.window > 0 ? row_pos[rt] - p.window + 1 : 0;   // first visible key
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = k0 + 4 * g + i;
+          const bool vis = key <= hi && key >= lo && key >= kb;
+          sc[i] = vis ? s[rt][i] : -INFINITY;
+          mx = fmaxf(mx, sc[i]);
+        }
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
       mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-      const float new_max = fmaxf(run_max[rt], mx);
+      const float new_max = fmaxf(run_max[rt], mx * p.scale_log2);
       const float base = new_max == -INFINITY ? 0.f : new_max;
       const float alpha = fast_exp2(run_max[rt] - base);   // 0 while nothing was seen yet
       float psum = 0.f;
       bf16x4 pb;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float pv = fast_exp2(sc[i] - base);
+        const float pv = fast_exp2(fmaf(sc[i], p.scale_log2, -base));
         psum += pv;
         pb[i] = static_cast<bf16_t>(pv);
       }
