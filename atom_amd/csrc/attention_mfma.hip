@@ -317,6 +317,191 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
   }
 }
 
+// Decode for head sizes 32, 64, 128 and 256 with pages of a multiple of 8 keys: the same work items and the
+// same two products as above, 32 keys a step, with every load a whole-line, 16-bytes-a-lane, non-temporal
+// one.  Key rows reach the first product's A operand through the wave's LDS area as above, but row r of
+// the two operand tiles b = 0, 1 is key 8 (r / 4) + 4 b + r % 4 of the step: lane (row, g) is then left
+// with the scores of keys 8 g .. 8 g + 7, which is the k order of one v_mfma_f32_16x16x32_bf16 step of the
+// second product, and its V^T operand (8 consecutive keys of one d) is one 16-byte load from the value page.
+template <int D, int RT>
+__global__ void __launch_bounds__(kWave) attention_decode32_kernel(AttnParams p) {
+  constexpr int KCH = D / 32;      // k steps of the first product
+  constexpr int DT = D / 16;       // output tiles along d
+  constexpr int KP = D * 32 / 8 / kWave;   // 16-byte pieces of a step's 32 key rows per lane
+  constexpr int KLDS = D * 2 + 16;
+  __shared__ __attribute__((aligned(16))) char klds[32 * KLDS];
+  const int lane = threadIdx.x;
+  const int r16 = lane & 15;
+  const int g = lane >> 4;
+  const int group = p.hq / p.hkv;
+  const int seq = blockIdx.z + p.seq_offset;
+  const int kvh = blockIdx.y;
+  const int part = blockIdx.x;
+  const int ctx = p.ctx_lens[seq];
+  const int head0 = kvh * group;
+  const int tok0 = p.cu_q[seq];
+  const int pos0 = ctx - 1;
+  const int* table = p.block_tables + (size_t)seq * p.max_blocks;
+  const int ps = p.page_size;
+
+  int vis0 = 0;
+  if (p.window > 0 && ctx - p.window > 0) vis0 = (ctx - p.window) & ~31;
+  int chunk = (ctx - vis0 + p.parts - 1) / p.parts;
+  chunk = (chunk + 31) & ~31;
+  const int kb = vis0 + part * chunk;
+  const int ke = min(ctx, kb + chunk);
+
+  bool row_ok[RT];
+  bf16x8 q32[RT][KCH];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = rt * 16 + r16;
+    row_ok[rt] = row < group;
+    const bf16_t* qr = p.q + ((size_t)tok0 * p.hq + head0 + row) * D;
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (row_ok[rt]) v = *reinterpret_cast<const bf16x8*>(qr + 32 * j + 8 * g);
+      q32[rt][j] = v;
+    }
+  }
+  f32x4 acc[RT][DT];
+  float run_max[RT], run_sum[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    run_max[rt] = -INFINITY;
+    run_sum[rt] = 0.f;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) acc[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  struct Step {
+    bf16x8 k[KP];
+    bf16x8 v[DT];
+  };
+  auto load_step = [&](int k0, Step& st) {
+#pragma unroll
+    for (int j = 0; j < KP; ++j) {
+      const int q = kWave * j + lane;                        // piece q: key q / (D / 8), elements (q % (D / 8)) * 8 ..
+      const int row = min(k0 + q / (D / 8), ke - 1);
+      const int page = table[row / ps];
+      st.k[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(
+          p.k_cache + (((size_t)page * p.hkv + kvh) * ps + (row % ps)) * D + (q % (D / 8)) * 8));
+    }
+    // this lane's keys of V^T are k0 + 8 g .. + 7 (one page: pages hold a multiple of 8 keys), rows d = 16 t + r16
+    const int vkey = min(k0 + 8 * g, (ke - 1) & ~7);
+    const int vpage = table[vkey / ps];
+    const bf16_t* vptr = p.v_cache + (((size_t)vpage * p.hkv + kvh) * D + r16) * (size_t)ps + (vkey % ps);
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+      st.v[t] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(vptr + (size_t)(16 * t) * ps));
+  };
+
+  Step cur, nxt;
+  if (kb < ke) load_step(kb, cur);
+  for (int k0 = kb; k0 < ke; k0 += 32) {
+    if (k0 + 32 < ke) load_step(k0 + 32, nxt);
+#pragma unroll
+    for (int j = 0; j < KP; ++j) {
+      const int q = kWave * j + lane;
+      *reinterpret_cast<bf16x8*>(klds + (q / (D / 8)) * KLDS + (q % (D / 8)) * 16) = cur.k[j];
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0); the block is one wave
+    __builtin_amdgcn_wave_barrier();
+    f32x4 s[RT][2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const char* krow = klds + (8 * (r16 / 4) + 4 * b + (r16 % 4)) * KLDS + 16 * g;
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(krow + 64 * j);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q32[rt][j], s[rt][b], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- softmax update; lane holds keys k0 + 8 g + 4 b + i of row r16
+    const bool whole = k0 + 31 <= ke - 1 && (p.window <= 0 || k0 >= pos0 - p.window + 1);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float sc[8];
+      float mx = -INFINITY;
+      if (whole) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          sc[e] = s[rt][e / 4][e % 4];
+          mx = fmaxf(mx, sc[e]);
+        }
+      } else {
+        const int lo = p.window > 0 ? pos0 - p.window + 1 : 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int key = k0 + 8 * g + e;
+          const bool vis = key < ke && key >= lo;
+          sc[e] = vis ? s[rt][e / 4][e % 4] : -INFINITY;
+          mx = fmaxf(mx, sc[e]);
+        }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float new_max = fmaxf(run_max[rt], mx * p.scale_log2);
+      const float base = new_max == -INFINITY ? 0.f : new_max;
+      const float alpha = fast_exp2(run_max[rt] - base);
+      float psum = 0.f;
+      bf16x8 pb;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float pv = fast_exp2(fmaf(sc[e], p.scale_log2, -base));
+        psum += pv;
+        pb[e] = static_cast<bf16_t>(pv);
+      }
+      run_sum[rt] = run_sum[rt] * alpha + psum;
+      run_max[rt] = new_max;
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        f32x4 a = acc[rt][t];
+        a[0] *= alpha; a[1] *= alpha; a[2] *= alpha; a[3] *= alpha;
+        acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.v[t], pb, a, 0, 0, 0);
+      }
+    }
+    cur = nxt;
+  }
+
+  // ---- write: lane holds O[row r16][d = 16 t + 4 g + i]
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    float total = run_sum[rt];
+    total += __shfl_xor(total, 16, kWave);
+    total += __shfl_xor(total, 32, kWave);
+    if (!row_ok[rt]) continue;
+    const int row = rt * 16 + r16;
+    if (p.parts > 1) {
+      const size_t slot = ((size_t)(blockIdx.z * p.hq + head0 + row)) * p.parts + part;
+      float* wo = p.ws_o + slot * D;
+#pragma unroll
+      for (int t = 0; t < DT; ++t) *reinterpret_cast<f32x4*>(wo + 16 * t + 4 * g) = acc[rt][t];
+      if (g == 0) {
+        p.ws_ml[slot * 2] = run_max[rt];
+        p.ws_ml[slot * 2 + 1] = total;
+      }
+    } else {
+      bf16_t* dst = p.out + ((size_t)tok0 * p.hq + head0 + row) * D;
+      const float inv = total > 0.f ? 1.f / total : 0.f;
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        bf16x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = static_cast<bf16_t>(acc[rt][t][i] * inv);
+        *reinterpret_cast<bf16x4*>(dst + 16 * t + 4 * g) = o;
+      }
+    }
+  }
+}
+
 // Merges the partial results of a decode row: one block of kMergeGroups waves per (request, head).
 // Lane k of every wave first holds the weight of part k (parts <= 64).  Wave w then adds the
 // parts w, w + kMergeGroups, ... (all their loads are issued together) and the waves' sums are
@@ -373,9 +558,20 @@ template <int D>
 static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
   const int group = p.hq / p.hkv;
   dim3 grid(p.parts, p.hkv, seqs), block(kWave);
-  if (group <= 16) hipLaunchKernelGGL((attention_mfma_kernel<D, 1, true>), grid, block, 0, stream, p);
-  else if (group <= 32) hipLaunchKernelGGL((attention_mfma_kernel<D, 2, true>), grid, block, 0, stream, p);
-  else return ATOM_UNSUPPORTED;
+  constexpr bool LINES = D == 32 || D == 64 || D == 128 || D == 256;
+  if (group > 32) return ATOM_UNSUPPORTED;
+  if constexpr (LINES) {
+    if (p.page_size % 8 == 0) {
+      if (group <= 16) hipLaunchKernelGGL((attention_decode32_kernel<D, 1>), grid, block, 0, stream, p);
+      else hipLaunchKernelGGL((attention_decode32_kernel<D, 2>), grid, block, 0, stream, p);
+    } else {
+      if (group <= 16) hipLaunchKernelGGL((attention_mfma_kernel<D, 1, true>), grid, block, 0, stream, p);
+      else hipLaunchKernelGGL((attention_mfma_kernel<D, 2, true>), grid, block, 0, stream, p);
+    }
+  } else {
+    if (group <= 16) hipLaunchKernelGGL((attention_mfma_kernel<D, 1, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((attention_mfma_kernel<D, 2, true>), grid, block, 0, stream, p);
+  }
   if (p.parts > 1)
     hipLaunchKernelGGL(attention_merge_kernel, dim3(p.hq, seqs), dim3(kMergeGroups * kWave), 0, stream, p.ws_o,
                        p.ws_ml, p.out, p.cu_q, p.seq_offset, p.hq, D, p.parts);
