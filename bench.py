@@ -58,6 +58,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
+    ap.add_argument("--max-model-len", type=int, default=None,
+                    help="positions a request may reach (default: 4096, or twice a longer --context)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--points", type=str, default="1,64", help="other decode batch sizes to time")
     ap.add_argument("--no-prefill", action="store_true")
@@ -85,7 +87,7 @@ def main() -> int:
     points = sorted({int(x) for x in args.points.split(",") if x} | {args.batch})
     points = [p for p in points]
     max_seqs = max(points + [args.mixed])
-    max_model_len = 4096
+    max_model_len = args.max_model_len or max(4096, 2 * args.context)
     block = 16
     t0 = time.time()
     llm = LLMEngine("qwen3-8b-random", model_config=cfg, load_dummy="random", seed=2, dtype="bf16",
