@@ -42,10 +42,24 @@ struct AttnParams {
   float* ws_o;            // decode: [seqs, Hq, parts, D]
   float* ws_ml;           // decode: [seqs, Hq, parts, 2]
   int max_blocks, hq, hkv, page_size, window, seq_offset, parts, num_tiles;
+  int page_shift;         // log2(page_size) where that is a power of two, else -1
   float scale_log2;       // softmax scale * log2(e)
 };
 
 __device__ __forceinline__ s16x4 as_s16x4(bf16x4 v) { return __builtin_bit_cast(s16x4, v); }
+
+// Where a key lies: its page's place in the block table and its place in the page.  A power-of-two
+// page size (the usual case) makes these a shift and a mask instead of a division per load.
+// The choice is made once per group of loads (POW2 is a compile-time constant), never per load: a branch
+// between a table look-up and the load that depends on it keeps the loads of a group from being in flight together.
+template <bool POW2>
+struct PageMath {
+  int size, shift;
+  __device__ __forceinline__ int index(int key) const { return POW2 ? key >> shift : key / size; }
+  __device__ __forceinline__ int within(int key) const { return POW2 ? key & (size - 1) : key % size; }
+};
+struct Pow2Pages { static constexpr bool value = true; };
+struct AnyPages { static constexpr bool value = false; };
 
 // 2^x for x <= 0 (and -inf): the bare instruction.  Results below the smallest normal number become 0,
 // which a probability may.
@@ -379,22 +393,29 @@ __global__ void __launch_bounds__(kWave) attention_decode32_kernel(AttnParams p)
     bf16x8 k[KP];
     bf16x8 v[DT];
   };
-  auto load_step = [&](int k0, Step& st) {
+  const size_t page_elems = (size_t)p.hkv * ps * D;        // elements of a page, all heads
+  const int k_head = kvh * ps * D, v_head = kvh * D * ps;
+  auto load_step_as = [&](int k0, Step& st, auto kind) {
+    const PageMath<decltype(kind)::value> pages{ps, p.page_shift};
 #pragma unroll
     for (int j = 0; j < KP; ++j) {
       const int q = kWave * j + lane;                        // piece q: key q / (D / 8), elements (q % (D / 8)) * 8 ..
       const int row = min(k0 + q / (D / 8), ke - 1);
-      const int page = table[row / ps];
+      const int page = table[pages.index(row)];
       st.k[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(
-          p.k_cache + (((size_t)page * p.hkv + kvh) * ps + (row % ps)) * D + (q % (D / 8)) * 8));
+          p.k_cache + page * page_elems + (k_head + pages.within(row) * D + (q % (D / 8)) * 8)));
     }
     // this lane's keys of V^T are k0 + 8 g .. + 7 (one page: pages hold a multiple of 8 keys), rows d = 16 t + r16
     const int vkey = min(k0 + 8 * g, (ke - 1) & ~7);
-    const int vpage = table[vkey / ps];
-    const bf16_t* vptr = p.v_cache + (((size_t)vpage * p.hkv + kvh) * D + r16) * (size_t)ps + (vkey % ps);
+    const int vpage = table[pages.index(vkey)];
+    const bf16_t* vptr = p.v_cache + vpage * page_elems + (v_head + r16 * ps + pages.within(vkey));
 #pragma unroll
     for (int t = 0; t < DT; ++t)
       st.v[t] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(vptr + (size_t)(16 * t) * ps));
+  };
+  auto load_step = [&](int k0, Step& st) {
+    if (p.page_shift >= 0) load_step_as(k0, st, Pow2Pages{});
+    else load_step_as(k0, st, AnyPages{});
   };
 
   Step cur, nxt;
@@ -554,6 +575,13 @@ attention_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__
   }
 }
 
+static int page_shift_of(int page_size) {
+  if (page_size <= 0 || (page_size & (page_size - 1))) return -1;
+  int shift = 0;
+  while ((1 << shift) < page_size) ++shift;
+  return shift;
+}
+
 template <int D>
 static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
   const int group = p.hq / p.hkv;
@@ -680,20 +708,27 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
   // ---- moving a tile: piece q of K is (key q / (D/8), 8 elements at (q % (D/8)) * 8);
   //      piece q of V^T is (d = q / (TK/8), the 8 keys at (q % (TK/8)) * 8)
   bf16x8 kreg[PT], vreg[PT];
-  auto load_tile = [&](int k0) {
+  const size_t page_elems = (size_t)p.hkv * ps * D;        // elements of a page, all heads
+  const int k_head = kvh * ps * D, v_head = kvh * D * ps;  // this KV head's part of a key page and of a value page
+  auto load_tile_as = [&](int k0, auto kind) {
+    const PageMath<decltype(kind)::value> pages{ps, p.page_shift};
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
       const int q = tid + 256 * j;
       const int key = min(k0 + q / (D / 8), ke - 1);
-      const int page = table[key / ps];
-      kreg[j] = *reinterpret_cast<const bf16x8*>(p.k_cache + (((size_t)page * p.hkv + kvh) * ps + key % ps) * D +
-                                                 (q % (D / 8)) * 8);
+      const int page = table[pages.index(key)];
+      kreg[j] = *reinterpret_cast<const bf16x8*>(p.k_cache + page * page_elems +
+                                                 (k_head + pages.within(key) * D + (q % (D / 8)) * 8));
       const int d = q / (TK / 8);
       const int vkey = min(k0 + (q % (TK / 8)) * 8, (ke - 1) & ~7);
-      const int vpage = table[vkey / ps];
-      vreg[j] = *reinterpret_cast<const bf16x8*>(p.v_cache + (((size_t)vpage * p.hkv + kvh) * D + d) * (size_t)ps +
-                                                 vkey % ps);
+      const int vpage = table[pages.index(vkey)];
+      vreg[j] = *reinterpret_cast<const bf16x8*>(p.v_cache + vpage * page_elems +
+                                                 (v_head + d * ps + pages.within(vkey)));
     }
+  };
+  auto load_tile = [&](int k0) {
+    if (p.page_shift >= 0) load_tile_as(k0, Pow2Pages{});
+    else load_tile_as(k0, AnyPages{});
   };
   auto store_tile = [&]() {
 #pragma unroll
@@ -902,6 +937,7 @@ ATOM_EXPORT int atom_attention_decode(const void* q, const void* k_cache, const 
   p.out = (bf16_t*)out; p.cu_q = cu_q; p.ctx_lens = ctx_lens; p.block_tables = block_tables; p.tiles = nullptr;
   p.ws_o = ws_o; p.ws_ml = ws_ml; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
   p.window = window; p.seq_offset = seq_offset; p.parts = parts; p.scale_log2 = scale * 1.4426950408889634f;
+  p.page_shift = page_shift_of(page_size);
 #define CALL(DD) return launch_decode<DD>(p, seqs, stream)
   ATOM_FOR_HEAD_DIM(d, CALL)
 #undef CALL
@@ -922,6 +958,7 @@ ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const
   p.out = (bf16_t*)out; p.cu_q = cu_q; p.ctx_lens = ctx_lens; p.block_tables = block_tables; p.tiles = tiles;
   p.ws_o = nullptr; p.ws_ml = nullptr; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
   p.window = window; p.seq_offset = 0; p.parts = 1; p.scale_log2 = scale * 1.4426950408889634f;
+  p.page_shift = page_shift_of(page_size);
   p.num_tiles = num_tiles;
   if (tiled) {   // tiles of atom_attention_prefill_tile_rows() tokens for the kernel with shared key tiles
     if (!atom_attention_prefill_tile_rows(d, page_size, hq / hkv)) return ATOM_UNSUPPORTED;
