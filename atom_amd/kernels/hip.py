@@ -104,6 +104,7 @@ class HipKernels:
             raise KernelError(
                 "atom_amd runs on an AMD GPU only: torch.cuda.is_available() is False and there is no CPU path")
         self.device = torch.device(device)
+        self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         path = _build.build()
         try:
             self.lib = ctypes.CDLL(path)
@@ -169,22 +170,32 @@ class HipKernels:
     # ------------------------------------------------------------------ helpers
 
     def _stream(self):
-        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        # the current stream's handle, the short way: these few calls are made hundreds of times a step
+        return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(self._device_index))
 
     def _check(self, name: str, t: torch.Tensor, dtype=None, shape=None):
+        """Every operand of every call goes through here (a step makes over a thousand such calls):
+        the passing case costs a few attribute reads, the failing one says what is wrong."""
         if not isinstance(t, torch.Tensor):
             raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
-        if t.device.type != "cuda":
+        if not t.is_cuda:
             raise KernelError(f"{name}: must live on the GPU, is on {t.device}")
         if not t.is_contiguous():
             raise KernelError(f"{name}: must be contiguous (shape {tuple(t.shape)}, strides {t.stride()})")
         if dtype is not None:
-            allowed = dtype if isinstance(dtype, (tuple, list)) else (dtype,)
-            if t.dtype not in allowed:
-                raise KernelError(f"{name}: element type {t.dtype} not in {allowed}")
+            have = t.dtype
+            if have is not dtype and (not isinstance(dtype, (tuple, list)) or have not in dtype):
+                raise KernelError(f"{name}: element type {have} not in {dtype}")
         if shape is not None:
-            if len(shape) != t.dim() or any(s is not None and s != a for s, a in zip(shape, t.shape)):
-                raise KernelError(f"{name}: shape {tuple(t.shape)} does not match {tuple(shape)}")
+            have = t.shape
+            ok = len(shape) == len(have)
+            if ok:
+                for want, got in zip(shape, have):
+                    if want is not None and want != got:
+                        ok = False
+                        break
+            if not ok:
+                raise KernelError(f"{name}: shape {tuple(have)} does not match {tuple(shape)}")
         return t
 
     def _done(self, what: str, status: int):
