@@ -337,20 +337,27 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
 // the two operand tiles b = 0, 1 is key 8 (r / 4) + 4 b + r % 4 of the step: lane (row, g) is then left
 // with the scores of keys 8 g .. 8 g + 7, which is the k order of one v_mfma_f32_16x16x32_bf16 step of the
 // second product, and its V^T operand (8 consecutive keys of one d) is one 16-byte load from the value page.
-template <int D, int RT>
-__global__ void __launch_bounds__(kWave) attention_decode32_kernel(AttnParams p) {
+//
+// TOGETHER: the parts of a (request, KV head) are the waves of one block (at most 8: two waves a SIMD is what
+// the registers allow), which merges their results through LDS and writes the output itself; no second kernel
+// and no partial results in memory.  Otherwise a block is one wave and the merge kernel follows.
+template <int D, int RT, bool TOGETHER>
+__global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave) attention_decode32_kernel(AttnParams p) {
   constexpr int KCH = D / 32;      // k steps of the first product
   constexpr int DT = D / 16;       // output tiles along d
   constexpr int KP = D * 32 / 8 / kWave;   // 16-byte pieces of a step's 32 key rows per lane
   constexpr int KLDS = D * 2 + 16;
-  __shared__ __attribute__((aligned(16))) char klds[32 * KLDS];
-  const int lane = threadIdx.x;
+  constexpr int AREA = 32 * KLDS;  // LDS bytes of a wave: the key rows of a step, later its result
+  extern __shared__ __attribute__((aligned(16))) char decode_lds[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  char* klds = decode_lds + wave * AREA;
   const int r16 = lane & 15;
   const int g = lane >> 4;
   const int group = p.hq / p.hkv;
   const int seq = blockIdx.z + p.seq_offset;
   const int kvh = blockIdx.y;
-  const int part = blockIdx.x;
+  const int part = TOGETHER ? wave : blockIdx.x;
   const int ctx = p.ctx_lens[seq];
   const int head0 = kvh * group;
   const int tok0 = p.cu_q[seq];
@@ -492,6 +499,45 @@ __global__ void __launch_bounds__(kWave) attention_decode32_kernel(AttnParams p)
     cur = nxt;
   }
 
+  if constexpr (TOGETHER) {
+    // ---- every wave leaves its rows' (unnormalised output, maximum, sum) in its LDS area; then all threads
+    //      share the elements of the output: parts are added in part order
+    constexpr int ROWS = 16 * RT;
+    float* mine = reinterpret_cast<float*>(klds);          // [ROWS][D] then [ROWS] maxima then [ROWS] sums
+    static_assert(!TOGETHER || (ROWS * D + 2 * ROWS) * 4 <= AREA, "a wave's result must fit where its key rows were");
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float total = run_sum[rt];
+      total += __shfl_xor(total, 16, kWave);
+      total += __shfl_xor(total, 32, kWave);
+      const int row = rt * 16 + r16;
+#pragma unroll
+      for (int t = 0; t < DT; ++t) *reinterpret_cast<f32x4*>(mine + row * D + 16 * t + 4 * g) = acc[rt][t];
+      if (g == 0) {
+        mine[ROWS * D + row] = run_max[rt];
+        mine[ROWS * D + ROWS + row] = total;
+      }
+    }
+    __syncthreads();
+    const int parts = p.parts;
+    for (int item = threadIdx.x; item < group * D; item += blockDim.x) {
+      const int row = item / D, dd = item - row * D;
+      float top = -INFINITY;
+      for (int k = 0; k < parts; ++k)
+        top = fmaxf(top, reinterpret_cast<const float*>(decode_lds + k * AREA)[ROWS * D + row]);
+      float num = 0.f, den = 0.f;
+      for (int k = 0; k < parts; ++k) {
+        const float* theirs = reinterpret_cast<const float*>(decode_lds + k * AREA);
+        const float m = theirs[ROWS * D + row];
+        const float w = m == -INFINITY ? 0.f : fast_exp2(m - top);
+        den += w * theirs[ROWS * D + ROWS + row];
+        num += w * theirs[row * D + dd];
+      }
+      p.out[((size_t)tok0 * p.hq + head0 + row) * D + dd] = static_cast<bf16_t>(den > 0.f ? num / den : 0.f);
+    }
+    return;
+  }
+
   // ---- write: lane holds O[row r16][d = 16 t + 4 g + i]
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
@@ -590,8 +636,21 @@ static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
   if (group > 32) return ATOM_UNSUPPORTED;
   if constexpr (LINES) {
     if (p.page_size % 8 == 0) {
-      if (group <= 16) hipLaunchKernelGGL((attention_decode32_kernel<D, 1>), grid, block, 0, stream, p);
-      else hipLaunchKernelGGL((attention_decode32_kernel<D, 2>), grid, block, 0, stream, p);
+      constexpr size_t area = 32 * (D * 2 + 16);   // LDS bytes of a wave
+      if (p.parts > 1 && p.parts <= 8 && group <= 16) {
+        // the parts of a (request, KV head) as the waves of one block, which merges them itself
+        // (up to 16 heads a KV head: their results fit where a wave kept its key rows)
+        static bool allowed = false;
+        if (!allowed && hipFuncSetAttribute((const void*)attention_decode32_kernel<D, 1, true>,
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 8 * area) != hipSuccess)
+          return ATOM_LAUNCH_FAILED;
+        allowed = true;
+        hipLaunchKernelGGL((attention_decode32_kernel<D, 1, true>), dim3(1, p.hkv, seqs), dim3(p.parts * kWave),
+                           area * p.parts, stream, p);
+        return launch_status();
+      }
+      if (group <= 16) hipLaunchKernelGGL((attention_decode32_kernel<D, 1, false>), grid, block, area, stream, p);
+      else hipLaunchKernelGGL((attention_decode32_kernel<D, 2, false>), grid, block, area, stream, p);
     } else {
       if (group <= 16) hipLaunchKernelGGL((attention_mfma_kernel<D, 1, true>), grid, block, 0, stream, p);
       else hipLaunchKernelGGL((attention_mfma_kernel<D, 2, true>), grid, block, 0, stream, p);

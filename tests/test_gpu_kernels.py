@@ -321,6 +321,23 @@ def test_decode_split_over_waves(parts, window):
     close(out, want, torch.bfloat16)
 
 
+@pytest.mark.parametrize("hq,hkv,d,page", [(6, 3, 32, 8), (16, 1, 64, 24), (40, 2, 64, 16), (3, 1, 256, 32), (4, 4, 128, 16),
+                                             (5, 5, 96, 4)])
+@pytest.mark.parametrize("parts", [3, 8, 9])
+def test_decode_parts_in_one_block_or_merged(hq, hkv, d, page, parts):
+    """Up to 8 parts of a request with up to 16 heads a KV head are the waves of one block, which merges
+    them itself; more parts, larger groups and other head or page sizes go through the merge kernel."""
+    q_lens = [1, 1, 1, 1]
+    ctx_lens = [1, 33, 260, 1100]
+    for window in (None, 200):
+        q, kc, vc, meta = _attention_case(torch.bfloat16, hq, hkv, d, page, window, q_lens, ctx_lens, seed=hq + parts)
+        out = torch.empty_like(q, device=DEV)
+        gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, window, parts=parts)
+        want = torch.empty_like(q)
+        PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, window)
+        close(out, want, torch.bfloat16)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_far_key_among_hundreds(dtype):
     """One key far back carries nearly all the weight: an attention that drops or misplaces it
