@@ -167,3 +167,47 @@ def test_pages_filled_by_steps_launched_ahead_are_found_under_their_real_tokens(
         [longer], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))[0]
     assert again["token_ids"] == fresh["token_ids"]
     _idle(ahead)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_steps_launched_ahead_under_random_load(seed):
+    """Requests of random lengths and token counts arrive while others run, some end on a token, the pool
+    is small enough to preempt, prompts share beginnings (prefix cache): with and without steps
+    launched ahead every request gets the same tokens, and the cache's books stay right after every step."""
+    import random
+    from atom_amd import SamplingParams
+
+    rng = random.Random(seed)
+    shared = random_ids("A", 24, 500 + seed)
+    arrivals = []
+    for k in range(14):
+        body = random_ids("A", rng.randrange(1, 30), 600 + 20 * seed + k)
+        prompt = (shared[:rng.choice([0, 16, 24])] + body)[:60]
+        sp = SamplingParams(temperature=rng.choice([0.0, 0.0, 0.8]), max_tokens=rng.randrange(1, 40), seed=k,
+                            ignore_eos=rng.random() < 0.5)
+        arrivals.append((rng.randrange(0, 25), prompt, sp))
+    arrivals.sort(key=lambda a: a[0])
+
+    def run(deferred):
+        llm = _engine(deferred, "A", num_kvcache_blocks=6, max_num_seqs=3, eos_token_id=7, max_model_len=128,
+                      stop_token_ids=list(range(0, 256, 16)))
+        seqs, outputs, pending, step = {}, {}, list(arrivals), 0
+        while pending or not llm.is_finished():
+            while pending and pending[0][0] <= step:
+                _, prompt, sp = pending.pop(0)
+                seq = llm.add_request(prompt, sp)[0]
+                seqs[seq.id] = len(seqs)
+            for seq in llm.step():
+                outputs[seqs[seq.id]] = (seq.completion_token_ids, seq.leave_reason)
+            llm.core.manager.check()
+            step += 1
+            assert step < 2000
+        _idle(llm)
+        return outputs, llm
+
+    waited, _ = run(False)
+    ahead, llm = run(True)
+    assert len(waited) == len(arrivals) and ahead == waited
+    reasons = [reason for _, reason in ahead.values()]
+    assert any(r.startswith("stop_") or r == "eos" for r in reasons) and "max_tokens" in reasons
+    assert llm.scheduler.total_preemptions > 0 and llm.core.manager.pools[0].hits > 0
