@@ -5,7 +5,7 @@ architecture; an architecture is a function from its configuration to a ``ModelS
 
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 
 import torch
 

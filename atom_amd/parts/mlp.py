@@ -4,8 +4,6 @@ atom/model_ops/activation.py:78-82)."""
 
 from __future__ import annotations
 
-import torch
-
 from .base import FEED_FORWARDS, FeedForward, ParamSpec
 
 

@@ -15,7 +15,7 @@ from __future__ import annotations
 
 import json
 import os
-from typing import Callable, Iterable
+from typing import Callable
 
 import torch
 

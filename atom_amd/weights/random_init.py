@@ -19,7 +19,7 @@ import torch
 
 from ..config.model_config import ModelConfig
 from ..config.registry import build_model
-from .loader import DictSource, TensorSource, expected_tensors
+from .loader import TensorSource, expected_tensors
 
 
 def random_tensor(name: str, shape, init: str, seed: int, std: float, norm_std: float,

@@ -12,7 +12,6 @@ library routine or an invariant (see ``test_plain_model.py``).
 from __future__ import annotations
 
 import json
-import math
 import os
 
 import torch

@@ -4,7 +4,6 @@ must reproduce the plain implementation under every way of cutting the work.  Wh
 tested here is paging, batching and metadata; the kernels themselves are tested on the GPU."""
 
 import pytest
-import torch
 
 import replay
 from helpers import make_core, oracle_logits, random_ids

@@ -18,7 +18,7 @@ from atom_amd.engine.context import KVBinding, StepContext
 from atom_amd.engine.core import StepEntry, build_core, load_model
 from atom_amd.kernels.hip import AttentionMeta
 from atom_amd.models.model import ModelSpec
-from atom_amd.parts import (FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, FeedForward, GatedMLP,
+from atom_amd.parts import (FEED_FORWARDS, MIXERS, POSITION_ENCODINGS, FeedForward, GatedMLP,
                             GroupedQueryAttention, LMHead, Mixer, ParamSpec, PartChoice, PositionEncoding, PreNormBlock,
                             RMSNorm, RotaryEncoding, StateNeed, TokenEmbedding)
 from atom_amd.weights import write_random_model

@@ -4,10 +4,7 @@ in portions of changing size, down to two tokens; and mixed, up to four live req
 with so few pages that they are used again.  Once in process on ``EngineCore`` and once
 through ``bin/trace_run``."""
 
-import os
-
 import pytest
-import torch
 
 import replay
 from helpers import gpu_ops, make_core, oracle_logits, random_ids, tiny_folder
