@@ -123,12 +123,21 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
 
     for (; kc < kc_end; kc += kSkinnyChunk) {
       const char* xb = smem + (kc - x0) * 2;
+      const bool more = kc + kSkinnyChunk < kc_end;
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4) {
         // a quarter of the shot into the operand layout through the wave's own LDS area
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg)
           *reinterpret_cast<bf16x8*>(mine + (4 * rg + g) * kARow + r16 * 16) = a[4 * s4 + rg];
+        if (more) {   // these four registers are free again: the same quarter of the next shot
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg) {
+            const int kk = kc + kSkinnyChunk + 128 * s4;
+            a[4 * s4 + rg] = (kk + 8 * r16 < k)
+                                 ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[rg] + kk)) : zero;
+          }
+        }
         __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the area is this wave's alone, no block barrier
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -143,7 +152,6 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
         __builtin_amdgcn_s_waitcnt(0xc07f);
         __builtin_amdgcn_wave_barrier();
       }
-      if (kc + kSkinnyChunk < kc_end) load_shot(kc + kSkinnyChunk);
     }
   }
 
