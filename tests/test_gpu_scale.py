@@ -131,3 +131,65 @@ def test_32_bit_and_bfloat16_agree_at_serving_sizes():
     half = _core(torch.bfloat16, num_pages=128, max_num_seqs=2).step([StepEntry("x", ids, want)]).cpu()
     _close(half, wide, "bfloat16", "bfloat16 against 32-bit")
     assert (half.argmax(-1) == wide.argmax(-1)).float().mean() >= 0.7
+
+
+def test_pages_far_into_a_large_cache():
+    """A cache of 140,000 pages (4.6 GB each for keys and values): pages whose offsets no 32-bit number
+    holds are written and read like the first ones (rotation + cache write, decode and prefill attention)."""
+    from atom_amd.kernels.hip import AttentionMeta
+
+    ops, dev = gpu_ops(), "cuda:0"
+    hq, hkv, d, page, base = 32, 8, 128, 16, 139_000
+    gen = torch.Generator().manual_seed(4)
+    lens = [1000, 37]            # two requests decode; a third brings a prompt portion of 300 tokens after 212 cached
+    pages_of = [63, 3, 32]
+    first = [0, 63, 66]
+
+    def run(offset, num_pages):
+        kc = torch.zeros(num_pages, hkv, page, d, dtype=torch.bfloat16, device=dev)
+        vc = torch.zeros(num_pages, hkv, d, page, dtype=torch.bfloat16, device=dev)
+        g = torch.Generator().manual_seed(4)
+        total = sum(pages_of)
+        kc[offset:offset + total] = (torch.randn(total, hkv, page, d, generator=g) * 0.5).to(torch.bfloat16).to(dev)
+        vc[offset:offset + total] = (torch.randn(total, hkv, d, page, generator=g) * 0.5).to(torch.bfloat16).to(dev)
+        tokens = 300 + 2
+        qkv = (torch.randn(tokens, (hq + 2 * hkv) * d, generator=g) * 0.5).to(torch.bfloat16).to(dev)
+        width = max(pages_of)
+        bt = torch.zeros(3, width, dtype=torch.int32)
+        for r in range(3):
+            bt[r, :pages_of[r]] = torch.arange(pages_of[r]) + offset + first[r]
+        # token order: the prompt portion first (request 2), then the two decode rows (requests 0 and 1)
+        order = [2, 0, 1]
+        bt = bt[order].contiguous().to(dev)
+        ctx = [512, lens[0], lens[1]]
+        positions = torch.tensor(list(range(212, 512)) + [lens[0] - 1, lens[1] - 1], dtype=torch.int32)
+        token_seq = torch.tensor([0] * 300 + [1, 2], dtype=torch.int32)
+        slots = torch.tensor([int(bt[s, p // page]) * page + p % page for s, p in zip(token_seq.tolist(), positions.tolist())],
+                             dtype=torch.int32).to(dev)
+        half = d // 2
+        inv = 1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        ang = torch.arange(1024, dtype=torch.float32)[:, None] * inv[None, :]
+        cos, sin = ang.cos().to(dev), ang.sin().to(dev)
+        w = torch.ones(d, device=dev)
+        q = torch.empty(tokens, hq, d, dtype=torch.bfloat16, device=dev)
+        ops.qk_norm_rope_kv_write(qkv, q, kc, vc, w, w, cos, sin, positions.to(dev), slots, hq, hkv, d, d, page, 1e-6)
+        tiles = {rows: torch.tensor([(0, r) for r in range(0, 300, rows)], dtype=torch.int32, device=dev)
+                 for rows in (32, 64, 128)}
+        meta = AttentionMeta(token_seq=token_seq.to(dev), positions=positions.to(dev), block_tables=bt,
+                             cu_seqlens_q=torch.tensor([0, 300, 301, 302], dtype=torch.int32, device=dev),
+                             context_lens=torch.tensor(ctx, dtype=torch.int32, device=dev), num_seqs=3, num_tokens=tokens,
+                             max_q_len=300, max_context_len=1000, page_size=page, num_prefill=1,
+                             prefill_tiles=tiles[32], rows_per_tile=32, tiles_by_rows=tiles)
+        out = torch.empty_like(q)
+        ops.paged_attention(q, kc, vc, out, meta, d ** -0.5)
+        torch.cuda.synchronize()
+        written = (kc[offset + first[2] + 13:offset + first[2] + 32].clone(), vc[offset + first[2] + 13:offset + first[2] + 32].clone())
+        return out.cpu(), written[0].cpu(), written[1].cpu()
+
+    low = run(0, 128)
+    torch.cuda.empty_cache()
+    high = run(base, base + 128)
+    assert (base + 100) * hkv * page * d > 2 ** 31
+    for a, b in zip(low, high):
+        assert torch.isfinite(a.float()).all() and torch.equal(a, b)
+    assert float(low[0].float().abs().max()) > 0 and float(low[1].float().abs().max()) > 0
