@@ -414,6 +414,22 @@ def test_sample_matches_plain_given_noise(top_k, top_p):
         assert out.cpu().tolist() == logits.argmax(dim=-1).tolist()
 
 
+@pytest.mark.parametrize("top_k,top_p", [(-1, 1.0), (50, 1.0), (-1, 0.8), (40, 0.95)])
+def test_sample_at_a_real_vocabulary(top_k, top_p):
+    """151,936 tokens: the filters and the race pick what the plain implementation picks."""
+    rows, vocab = 5, 151936
+    logits = rnd((rows, vocab), torch.float32, 41, 3.0)
+    temps = torch.tensor([0.7, 1.0, 0.0, 1.3, 0.6], dtype=torch.float32)
+    noise = torch.empty((rows, vocab)).exponential_(generator=torch.Generator().manual_seed(42))
+    ks = torch.full((rows,), top_k, dtype=torch.int32)
+    ps = torch.full((rows,), top_p, dtype=torch.float32)
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    gpu_ops().sample(logits.to(DEV), temps.to(DEV), out, top_ks=ks.to(DEV), top_ps=ps.to(DEV), noise=noise.to(DEV))
+    want = torch.empty(rows, dtype=torch.int32)
+    PLAIN.sample(logits, temps, want, top_ks=ks, top_ps=ps, noise=noise)
+    assert out.cpu().tolist() == want.tolist()
+
+
 def test_sample_frequencies_follow_softmax():
     vocab, draws = 11, 20000
     logits = torch.tensor([[2.0, 1.0, 0.5, 0.0, -1.0, 1.5, 0.2, -3.0, 0.9, 1.1, -0.5]])
