@@ -6,13 +6,15 @@
 //   top-k / top-p:           the race runs only among the kept tokens: the k likeliest, and of the
 //                            descending order those whose preceding mass is <= top_p (the likeliest
 //                            token always stays).  Both sets are "scaled logit >= threshold" sets, and
-//                            each threshold is found by a 32-step search over the bit pattern.
+//                            each threshold is found digit by digit (12, 12 and 8 bits of the logit's
+//                            order-preserving bit pattern) from histograms of counts and of mass.
 // The noise is either given ([rows, vocab], or one row shared by all with noise_stride 0) or made
 // from (seed, counter, token) of the row by an integer mix, so a request's draws do not depend on
 // what else is in the batch.
 #include "common.h"
 
 constexpr int kSampleThreads = 1024;
+constexpr int kDigitBins = 4096;   // bins of the widest digit of the threshold search
 
 __device__ __forceinline__ uint64_t mix64(uint64_t x) {
   x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
@@ -90,38 +92,96 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   const float p = top_ps ? top_ps[r] : 1.f;
   uint32_t threshold = 0u;  // keep keys >= threshold
 
-  if (k > 0 && k < vocab) {
-    // largest key u with count(key >= u) >= k
-    uint32_t u = 0u;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t cand = u | (1u << bit);
-      float cnt = 0.f;
-      for (int v = tid; v < vocab; v += kSampleThreads)
-        cnt += float_key((row[v] - top) * inv_t) >= cand ? 1.f : 0.f;
-      cnt = block_sum(cnt, scratch);
-      if (cnt >= (float)k) u = cand;
+  const bool want_k = k > 0 && k < vocab;
+  const bool want_p = p < 1.f;
+  if (want_k || want_p) {
+    // Two thresholds over key = float_key(scaled logit), found together, a digit a pass:
+    //   top-k  u_k = the k-th largest key: the largest u with count(key >= u) >= k
+    //   top-p  u_p = the smallest u with mass(key > u) <= p * total mass
+    // A pass builds, over the keys that share the digits found so far, a histogram of the next digit:
+    // counts for u_k, mass (exp of the scaled logit, as a 2^40 fixed-point integer, so that the sums do
+    // not depend on the order of the additions) for u_p.  One wave then walks the histogram from the top.
+    __shared__ unsigned int hist_cnt[kDigitBins];
+    __shared__ unsigned long long hist_mass[kDigitBins];
+    __shared__ unsigned int found_k, found_p;          // the digits found so far, as the key's top bits
+    __shared__ unsigned int left_k;                    // how many of the k are still to be found below
+    __shared__ unsigned long long left_mass;           // how much of the budget is left for what lies below
+    if (tid == 0) {
+      found_k = found_p = 0u;
+      left_k = want_k ? (unsigned int)k : 0u;
+      left_mass = 0ull;
     }
-    threshold = u;
-  }
-  if (p < 1.f) {
-    float z = 0.f;
-    for (int v = tid; v < vocab; v += kSampleThreads) z += expf((row[v] - top) * inv_t);
-    z = block_sum(z, scratch);
-    const float budget = p * z;
-    // smallest key u with mass(key > u) <= budget; the predicate is monotone in u
-    uint32_t u = 0u;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t cand = u | (1u << bit);
-      // test cand - 1: if mass above (cand - 1) is still over budget, the answer is >= cand
-      float mass = 0.f;
-      for (int v = tid; v < vocab; v += kSampleThreads) {
-        const float s = (row[v] - top) * inv_t;
-        mass += float_key(s) > cand - 1u ? expf(s) : 0.f;
+    const int shifts[3] = {20, 8, 0};
+    const int widths[3] = {12, 12, 8};
+    for (int pass = 0; pass < 3; ++pass) {
+      const int shift = shifts[pass], bins = 1 << widths[pass];
+      for (int b = tid; b < bins; b += kSampleThreads) {
+        hist_cnt[b] = 0u;
+        hist_mass[b] = 0ull;
       }
-      mass = block_sum(mass, scratch);
-      if (mass > budget) u = cand;
+      __syncthreads();
+      const unsigned int prefix_k = found_k, prefix_p = found_p;
+      const int above = shift + widths[pass];      // bits above this digit (32: none)
+      for (int v = tid; v < vocab; v += kSampleThreads) {
+        const float sl = (row[v] - top) * inv_t;
+        const uint32_t key = float_key(sl);
+        const uint32_t digit = (key >> shift) & (uint32_t)(bins - 1);
+        const uint32_t high = above >= 32 ? 0u : key >> above;
+        if (want_k && high == (above >= 32 ? 0u : prefix_k >> above)) atomicAdd(&hist_cnt[digit], 1u);
+        if (want_p && high == (above >= 32 ? 0u : prefix_p >> above))
+          atomicAdd(&hist_mass[digit], (unsigned long long)(expf(sl) * 1099511627776.f));
+      }
+      __syncthreads();
+      if (tid < kWave) {
+        // lane l owns bins [per * l, per * l + per): what lies in higher bins, then a walk down its own
+        const int per = bins / kWave;
+        unsigned int cnt_own = 0u;
+        unsigned long long mass_own = 0ull;
+        for (int b = 0; b < per; ++b) {
+          cnt_own += hist_cnt[per * tid + b];
+          mass_own += hist_mass[per * tid + b];
+        }
+        unsigned int cnt_above = cnt_own;
+        unsigned long long mass_above = mass_own;
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {   // inclusive sums over lanes >= this one
+          const unsigned int c = __shfl_down(cnt_above, off, kWave);
+          const unsigned long long m = __shfl_down(mass_above, off, kWave);
+          if (tid + off < kWave) {
+            cnt_above += c;
+            mass_above += m;
+          }
+        }
+        const unsigned long long total_mass = __shfl(mass_above, 0, kWave);
+        cnt_above -= cnt_own;
+        mass_above -= mass_own;
+        if (want_p && pass == 0 && tid == 0) left_mass = (unsigned long long)((double)p * (double)total_mass);
+        // (the budget is read by every lane after this point; it is written by lane 0 of this same wave)
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+        const unsigned int need = left_k;
+        const unsigned long long budget = left_mass;
+        for (int b = per - 1; b >= 0; --b) {
+          const int bin = per * tid + b;
+          const unsigned int c = hist_cnt[bin];
+          const unsigned long long m = hist_mass[bin];
+          if (want_k && cnt_above < need && cnt_above + c >= need) {   // the k-th largest lies in this bin
+            found_k = prefix_k | ((unsigned int)bin << shift);
+            left_k = need - cnt_above;
+          }
+          // the lowest bin whose higher bins hold no more than the budget
+          if (want_p && mass_above <= budget && (mass_above + m > budget || bin == 0)) {
+            found_p = prefix_p | ((unsigned int)bin << shift);
+            left_mass = budget - mass_above;
+          }
+          cnt_above += c;
+          mass_above += m;
+        }
+      }
+      __syncthreads();
     }
-    if (u > threshold) threshold = u;
+    if (want_k) threshold = found_k;
+    if (want_p && found_p > threshold) threshold = found_p;
   }
 
   const float* nrow = noise ? noise + (size_t)r * noise_stride : nullptr;
@@ -176,7 +236,53 @@ argmax_pick_kernel(const float* __restrict__ ws_vals, const int* __restrict__ ws
   if (threadIdx.x == 0) out[r] = m.i;
 }
 
-// `ws_vals` / `ws_idx` (rows * 64 elements each, or null) let all-greedy calls take the two-step path.
+// The exponential race of rows without top-k / top-p, over chunks: a block runs the race among the tokens of
+// one chunk of one row (the row's maximum is the largest of the chunks' maxima that argmax_chunks_kernel
+// left), and argmax_pick_kernel picks among the chunks' winners.  A row with temperature 0 hands its chunk's
+// maximum on.  Values and tie rule are sample_kernel's, so the token is the same.
+__global__ void __launch_bounds__(256)
+race_chunks_kernel(const float* __restrict__ logits, const float* __restrict__ temperatures,
+                   const float* __restrict__ noise, long noise_stride, const unsigned long long* __restrict__ seeds,
+                   const unsigned long long* __restrict__ counters, const float* __restrict__ max_vals,
+                   const int* __restrict__ max_idx, float* __restrict__ ws_vals, int* __restrict__ ws_idx, int vocab,
+                   float eps) {
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  const int r = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const float temp = temperatures[r];
+  if (!(temp > 0.f)) {
+    if (threadIdx.x == 0) {
+      ws_vals[r * kArgmaxChunks + chunk] = max_vals[r * kArgmaxChunks + chunk];
+      ws_idx[r * kArgmaxChunks + chunk] = max_idx[r * kArgmaxChunks + chunk];
+    }
+    return;
+  }
+  float top = max_vals[r * kArgmaxChunks + (threadIdx.x & (kWave - 1))];
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) top = fmaxf(top, __shfl_xor(top, off, kWave));
+  const int per = (vocab + kArgmaxChunks - 1) / kArgmaxChunks;
+  const int lo = chunk * per, hi = min(vocab, lo + per);
+  const float* row = logits + (size_t)r * vocab;
+  const float* nrow = noise ? noise + (size_t)r * noise_stride : nullptr;
+  const uint64_t seed = seeds ? seeds[r] : 0ull;
+  const uint64_t counter = counters ? counters[r] : 0ull;
+  const float inv_t = 1.f / temp;
+  MaxIdx best{-INFINITY, 0x7fffffff};
+  for (int v = lo + threadIdx.x; v < hi; v += blockDim.x) {
+    const float s = (row[v] - top) * inv_t;
+    const float e = nrow ? nrow[v] : exponential_draw(seed, counter, v);
+    best = better(best, MaxIdx{expf(s) / (e + eps), v});
+  }
+  best = block_argmax(best, sv, si);
+  if (threadIdx.x == 0) {
+    ws_vals[r * kArgmaxChunks + chunk] = best.v;
+    ws_idx[r * kArgmaxChunks + chunk] = best.i;
+  }
+}
+
+// `ws_vals` / `ws_idx` (rows * 128 elements each, or null) let calls without top-k / top-p spread every row
+// of a large vocabulary over 64 blocks.
 ATOM_EXPORT int atom_sample(const float* logits, const float* temperatures, const int* top_ks, const float* top_ps,
                             const float* noise, long noise_stride, const unsigned long long* seeds,
                             const unsigned long long* counters, int* out, int rows, int vocab, float eps,
@@ -184,10 +290,18 @@ ATOM_EXPORT int atom_sample(const float* logits, const float* temperatures, cons
   if (rows < 0 || vocab <= 0) return ATOM_BAD_SHAPE;
   if (rows == 0) return ATOM_OK;
   static_assert(kArgmaxChunks == kWave, "the pick kernel holds one chunk per lane");
-  if (!temperatures && ws_vals && ws_idx && vocab >= 16384 && rows <= 65535) {
+  if (!top_ks && !top_ps && ws_vals && ws_idx && vocab >= 16384 && rows <= 65535) {
     hipLaunchKernelGGL(argmax_chunks_kernel, dim3(kArgmaxChunks, rows), dim3(256), 0, stream, logits, ws_vals, ws_idx,
                        vocab);
-    hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(kWave), 0, stream, ws_vals, ws_idx, out);
+    if (temperatures) {   // the race among each chunk's tokens, into the second half of the workspaces
+      float* race_vals = ws_vals + (size_t)rows * kArgmaxChunks;
+      int* race_idx = ws_idx + (size_t)rows * kArgmaxChunks;
+      hipLaunchKernelGGL(race_chunks_kernel, dim3(kArgmaxChunks, rows), dim3(256), 0, stream, logits, temperatures,
+                         noise, noise_stride, seeds, counters, ws_vals, ws_idx, race_vals, race_idx, vocab, eps);
+      hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(kWave), 0, stream, race_vals, race_idx, out);
+    } else {
+      hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(kWave), 0, stream, ws_vals, ws_idx, out);
+    }
     return launch_status();
   }
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kSampleThreads), 0, stream, logits, temperatures, top_ks,
