@@ -103,7 +103,7 @@ class LLMEngine:
         if self.core.graphs is not None:   # as the reference's engine does before it serves (engine_core.py:131-138)
             self.core.graphs.capture_all()
         self.scheduler = Scheduler(cfg, self.core)
-        self.sampler = Sampler(ops, cfg.device)
+        self.sampler = Sampler(ops, cfg.device, cfg.max_num_seqs)
         self.seqs: dict[int, Sequence] = {}
         self._profiler = None
         self.deferred_output = bool(cfg.deferred_output)

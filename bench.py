@@ -66,6 +66,9 @@ def main() -> int:
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
                     help="instead: N requests with prompts of 64..3072 tokens through the scheduler, prompt portions of "
                          "512 tokens beside running decodes, 128 output tokens each; prints its own line")
+    ap.add_argument("--temperature", type=float, default=0.0, help="of the decode steps' sampling (0: greedy)")
+    ap.add_argument("--top-p", type=float, default=1.0)
+    ap.add_argument("--top-k", type=int, default=-1)
     ap.add_argument("--enforce-eager", action="store_true")
     ap.add_argument("--no-deferred-output", action="store_true",
                     help="read every step's tokens before the next step is launched")
@@ -152,7 +155,8 @@ def main() -> int:
         # prompts are admitted over several steps, so the first requests are some tokens ahead of the last
         # when all decode: leave room, so that none finishes (and the batch does not shrink) while timed
         admission_steps = -(-batch * args.context // 16384) + 1
-        sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + admission_steps + 2, ignore_eos=True)
+        sp = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, seed=1,
+                            max_tokens=steps + warmup + admission_steps + 2, ignore_eos=True)
         for _ in range(batch):
             llm.add_request(prompt(), sp)
         while any(s.num_completion_tokens == 0 for s in llm.seqs.values()):   # prompts, untimed
