@@ -15,6 +15,7 @@
 
 constexpr int kSampleThreads = 1024;
 constexpr int kDigitBins = 4096;   // bins of the widest digit of the threshold search
+constexpr int kArgmaxChunks = 64;  // blocks over which a row of a large vocabulary is spread
 
 __device__ __forceinline__ uint64_t mix64(uint64_t x) {
   x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
@@ -70,7 +71,8 @@ __global__ void __launch_bounds__(kSampleThreads)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperatures,
               const int* __restrict__ top_ks, const float* __restrict__ top_ps,
               const float* __restrict__ noise, long noise_stride, const unsigned long long* __restrict__ seeds,
-              const unsigned long long* __restrict__ counters, int* __restrict__ out, int vocab, float eps) {
+              const unsigned long long* __restrict__ counters, int* __restrict__ out, int vocab, float eps,
+              const float* __restrict__ chunk_vals, const int* __restrict__ chunk_idx) {
   __shared__ float sv[16];
   __shared__ int si[16];
   __shared__ float scratch[16];
@@ -79,8 +81,13 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   const float* row = logits + (size_t)r * vocab;
   const float temp = temperatures ? temperatures[r] : 0.f;
 
+  // the row's maximum: from the chunks' maxima where argmax_chunks_kernel has left them, else a scan
   MaxIdx m{-INFINITY, 0x7fffffff};
-  for (int v = tid; v < vocab; v += kSampleThreads) m = better(m, MaxIdx{row[v], v});
+  if (chunk_vals) {
+    if (tid < kArgmaxChunks) m = MaxIdx{chunk_vals[r * kArgmaxChunks + tid], chunk_idx[r * kArgmaxChunks + tid]};
+  } else {
+    for (int v = tid; v < vocab; v += kSampleThreads) m = better(m, MaxIdx{row[v], v});
+  }
   m = block_argmax(m, sv, si);
   if (!(temp > 0.f)) {
     if (tid == 0) out[r] = m.i;
@@ -201,8 +208,6 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
 // Greedy rows of a large vocabulary in two steps, so that a few rows still use the whole chip: every
 // block finds the maximum of one chunk of one row (lowest index on ties), then one wave per row picks
 // among the chunks' maxima, lowest chunk first.
-constexpr int kArgmaxChunks = 64;
-
 __global__ void __launch_bounds__(256)
 argmax_chunks_kernel(const float* __restrict__ logits, float* __restrict__ ws_vals, int* __restrict__ ws_idx,
                      int vocab) {
@@ -304,8 +309,13 @@ ATOM_EXPORT int atom_sample(const float* logits, const float* temperatures, cons
     }
     return launch_status();
   }
+  const bool spread = ws_vals && ws_idx && vocab >= 16384 && rows <= 65535;
+  if (spread)   // the rows' maxima by 64 blocks a row instead of one
+    hipLaunchKernelGGL(argmax_chunks_kernel, dim3(kArgmaxChunks, rows), dim3(256), 0, stream, logits, ws_vals, ws_idx,
+                       vocab);
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kSampleThreads), 0, stream, logits, temperatures, top_ks,
-                     top_ps, noise, noise_stride, seeds, counters, out, vocab, eps);
+                     top_ps, noise, noise_stride, seeds, counters, out, vocab, eps, spread ? ws_vals : nullptr,
+                     spread ? ws_idx : nullptr);
   return launch_status();
 }
 

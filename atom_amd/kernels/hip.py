@@ -477,10 +477,9 @@ class HipKernels:
         if seeds is not None:
             self._check("seeds", seeds, torch.int64, (rows,))
             self._check("counters", counters, torch.int64, (rows,))
-        ws_vals = ws_idx = None
-        if top_ks is None and top_ps is None:   # every row spread over 64 blocks: chunk maxima, then chunk winners
-            ws_vals = self.workspace("sample_vals", rows * 128)
-            ws_idx = self.workspace("sample_idx", rows * 128, torch.int32)
+        # every row's maximum (and, without filters, its race) is spread over 64 blocks: chunk maxima, chunk winners
+        ws_vals = self.workspace("sample_vals", rows * 128)
+        ws_idx = self.workspace("sample_idx", rows * 128, torch.int32)
         self._done("sample", self.lib.atom_sample(
             _ptr(logits), _ptr(temperatures), _ptr(top_ks), _ptr(top_ps), _ptr(noise), ctypes.c_long(stride),
             _ptr(seeds), _ptr(counters), _ptr(out), rows, vocab, ctypes.c_float(eps), _ptr(ws_vals), _ptr(ws_idx),
