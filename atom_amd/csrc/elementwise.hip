@@ -549,8 +549,61 @@ qk_norm_rope_vec_kernel(const T* __restrict__ qkv, T* __restrict__ q_out, T* __r
                         const float* __restrict__ q_weight, const float* __restrict__ k_weight,
                         const float* __restrict__ cos_table, const float* __restrict__ sin_table,
                         const int* __restrict__ positions, const int* __restrict__ slots, int tokens, int hq, int hkv,
-                        int page_size, float eps, int write_kv) {
+                        int page_size, float eps, int write_kv, T* __restrict__ v_cache, int qk_blocks) {
   constexpr int D = 16 * E;
+  if ((int)blockIdx.x >= qk_blocks) {
+    // ---- value heads: half a block (128 threads) takes 8 consecutive tokens of one KV head, lane i of token
+    //      j its E elements; the 8 x D tile goes through LDS so that, where the 8 slots are 8 consecutive
+    //      aligned places of one page, every d gets its 8 keys in one 16-byte store (value pages are
+    //      transposed).  Other groups (a prompt's ragged end, padding) scatter single elements.
+    __shared__ T tile[2][8][D];
+    const int half = threadIdx.x / 128, within = threadIdx.x % 128;
+    const int j = within / 16, vi = within & 15;
+    const int groups8 = (tokens + 7) / 8;
+    const int vg = ((int)blockIdx.x - qk_blocks) * 2 + half;
+    const bool group_live = vg < groups8 * hkv;
+    const int g8 = group_live ? vg / hkv : 0, kvh = group_live ? vg - g8 * hkv : 0;
+    const int t0 = 8 * g8, tv = t0 + j;
+    const size_t v_width = (size_t)(hq + 2 * hkv) * D;
+    constexpr int VALIGN = sizeof(T) * E < 16 ? sizeof(T) * E : 16;
+    T vals[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) vals[e] = from_f32<T>(0.f);
+    if (group_live && tv < tokens)
+      __builtin_memcpy(vals, __builtin_assume_aligned(qkv + (size_t)tv * v_width + (size_t)(hq + hkv + kvh) * D + E * vi,
+                                                      VALIGN), sizeof(vals));
+    bool together = group_live && t0 + 8 <= tokens && page_size % 8 == 0;
+    int s0 = -1;
+    if (together) {
+      s0 = slots[t0];
+      together = s0 >= 0 && s0 % 8 == 0;
+      for (int q = 1; q < 8 && together; ++q) together = slots[t0 + q] == s0 + q;
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) tile[half][j][E * vi + e] = vals[e];
+    __syncthreads();
+    if (!group_live) return;
+    if (together) {
+      const int page = s0 / page_size, off = s0 - page * page_size;
+      T* base = v_cache + ((size_t)page * hkv + kvh) * (size_t)D * page_size + off;
+      for (int dd = within; dd < D; dd += 128) {
+        T eight[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) eight[q] = tile[half][q][dd];
+        __builtin_memcpy(__builtin_assume_aligned(base + (size_t)dd * page_size, sizeof(T) * 8 < 16 ? sizeof(T) * 8 : 16),
+                         eight, sizeof(eight));
+      }
+    } else if (tv < tokens) {
+      const int slot = slots[tv];
+      if (slot >= 0) {
+        const int page = slot / page_size, off = slot - page * page_size;
+        T* dst = v_cache + ((size_t)page * hkv + kvh) * (size_t)D * page_size + off;
+#pragma unroll
+        for (int e = 0; e < E; ++e) dst[(size_t)(E * vi + e) * page_size] = vals[e];
+      }
+    }
+    return;
+  }
   const int pair = blockIdx.x * 16 + threadIdx.x / 16;
   const int i = threadIdx.x & 15;
   const int heads = hq + hkv;
@@ -618,14 +671,17 @@ ATOM_EXPORT int atom_qk_norm_rope_kv_write(
   int head_begin = 0;
   const long pairs = (long)tokens * (hq + hkv);
   if (!x_partial && tokens >= 32 && rotary_dim == d && d % 16 == 0 && d <= 256 && (d & (d - 1)) == 0 &&
-      pairs / 16 < 0x7fffffffL && (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache) & 31) == 0) {
-    // many tokens: q and k heads through the vector kernel, the value heads through the general one
-    const dim3 vgrid((unsigned)((pairs + 15) / 16)), vblock(256);
+      pairs / 16 + (long)tokens * hkv < 0x7fffffffL &&
+      (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)v_cache) & 31) == 0) {
+    // many tokens: q and k heads and, behind them in the same grid, the value heads through the vector kernel
+    const long qk_blocks = (pairs + 15) / 16;
+    const long v_blocks = write_kv ? ((long)((tokens + 7) / 8) * hkv + 1) / 2 : 0;
+    const dim3 vgrid((unsigned)(qk_blocks + v_blocks)), vblock(256);
 #define LAUNCH_ROPE(EE)                                                                                          \
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((qk_norm_rope_vec_kernel<T, EE>), vgrid, vblock, 0, stream,      \
                                                  (const T*)qkv, (T*)q_out, (T*)k_cache, q_weight, k_weight,      \
                                                  cos_table, sin_table, positions, slots, tokens, hq, hkv,        \
-                                                 page_size, eps, write_kv))
+                                                 page_size, eps, write_kv, (T*)v_cache, (int)qk_blocks))
     switch (d / 16) {
       case 1: LAUNCH_ROPE(1); break;
       case 2: LAUNCH_ROPE(2); break;
@@ -634,8 +690,7 @@ ATOM_EXPORT int atom_qk_norm_rope_kv_write(
       default: LAUNCH_ROPE(16); break;
     }
 #undef LAUNCH_ROPE
-    if (!write_kv) return launch_status();
-    head_begin = hq + hkv;
+    return launch_status();
   }
   dim3 grid(tokens, hq + 2 * hkv - head_begin), block(kWave);
   if ((size_t)d * 4 > 64 * 1024) return ATOM_TOO_LARGE;   // a head's values are kept in LDS
