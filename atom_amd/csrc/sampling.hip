@@ -250,11 +250,12 @@ race_chunks_kernel(const float* __restrict__ logits, const float* __restrict__ t
                    const float* __restrict__ noise, long noise_stride, const unsigned long long* __restrict__ seeds,
                    const unsigned long long* __restrict__ counters, const float* __restrict__ max_vals,
                    const int* __restrict__ max_idx, float* __restrict__ ws_vals, int* __restrict__ ws_idx, int vocab,
-                   float eps) {
+                   float eps, const unsigned int* __restrict__ thresholds) {
   __shared__ float sv[16];
   __shared__ int si[16];
   const int r = blockIdx.y;
   const int chunk = blockIdx.x;
+  const uint32_t threshold = thresholds ? thresholds[r] : 0u;   // only keys >= threshold take part
   const float temp = temperatures[r];
   if (!(temp > 0.f)) {
     if (threadIdx.x == 0) {
@@ -276,6 +277,7 @@ race_chunks_kernel(const float* __restrict__ logits, const float* __restrict__ t
   MaxIdx best{-INFINITY, 0x7fffffff};
   for (int v = lo + threadIdx.x; v < hi; v += blockDim.x) {
     const float s = (row[v] - top) * inv_t;
+    if (float_key(s) < threshold) continue;
     const float e = nrow ? nrow[v] : exponential_draw(seed, counter, v);
     best = better(best, MaxIdx{expf(s) / (e + eps), v});
   }
@@ -286,12 +288,175 @@ race_chunks_kernel(const float* __restrict__ logits, const float* __restrict__ t
   }
 }
 
+// ---- top-k / top-p thresholds of rows of a large vocabulary, spread over 64 blocks a row.
+//
+// The thresholds are those of sample_kernel (u_k: the k-th largest key; u_p: the smallest u with
+// mass(key > u) <= p * total mass; mass as a 2^40 fixed-point integer), found digit by digit (12, 12, 8 bits):
+// filter_hist_kernel adds a chunk's keys that share the digits found so far to the row's histogram of the next
+// digit (counts for u_k, mass for u_p), filter_select_kernel walks the histogram from the top, notes the digit
+// and what is left to find below it, and leaves the histogram zeroed for the next pass (and the next call: the
+// histograms must be zero when atom_sample is entered, and are when it returns).
+// state32[row] = {digits of u_k so far, what is left of k, digits of u_p so far, unused}; state64[row] = what is
+// left of the mass budget.
+struct FilterPass {
+  int shift, width;
+};
+__device__ __forceinline__ FilterPass filter_pass(int pass) {
+  return pass == 0 ? FilterPass{20, 12} : (pass == 1 ? FilterPass{8, 12} : FilterPass{0, 8});
+}
+
+template <int PASS>
+__global__ void __launch_bounds__(256)
+filter_hist_kernel(const float* __restrict__ logits, const float* __restrict__ temperatures,
+                   const int* __restrict__ top_ks, const float* __restrict__ top_ps,
+                   const float* __restrict__ max_vals, unsigned int* __restrict__ hist_cnt,
+                   unsigned long long* __restrict__ hist_mass, const unsigned int* __restrict__ state32, int vocab) {
+  const int r = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const float temp = temperatures[r];
+  const int k = top_ks ? top_ks[r] : -1;
+  const bool want_k = k > 0 && k < vocab;
+  const bool want_p = top_ps && top_ps[r] < 1.f;
+  if (!(temp > 0.f) || !(want_k || want_p)) return;
+  float top = max_vals[r * kArgmaxChunks + (threadIdx.x & (kWave - 1))];
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) top = fmaxf(top, __shfl_xor(top, off, kWave));
+  const FilterPass fp = filter_pass(PASS);
+  const int bins = 1 << fp.width, above = fp.shift + fp.width;
+  const uint32_t prefix_k = PASS ? state32[4 * r] >> above : 0u;
+  const uint32_t prefix_p = PASS ? state32[4 * r + 2] >> above : 0u;
+  const int per = (vocab + kArgmaxChunks - 1) / kArgmaxChunks;
+  const int lo = chunk * per, hi = min(vocab, lo + per);
+  const float* row = logits + (size_t)r * vocab;
+  const float inv_t = 1.f / temp;
+  unsigned int* cnt = hist_cnt + (size_t)r * kDigitBins;
+  unsigned long long* mass = hist_mass + (size_t)r * kDigitBins;
+  if (PASS == 0) {
+    // every key takes part: a histogram of the block in LDS first, then its non-empty bins to the row's
+    __shared__ unsigned int lcnt[kDigitBins];
+    __shared__ unsigned long long lmass[kDigitBins];
+    for (int b = threadIdx.x; b < bins; b += blockDim.x) {
+      lcnt[b] = 0u;
+      lmass[b] = 0ull;
+    }
+    __syncthreads();
+    for (int v = lo + threadIdx.x; v < hi; v += blockDim.x) {
+      const float sl = (row[v] - top) * inv_t;
+      const uint32_t digit = float_key(sl) >> fp.shift;
+      if (want_k) atomicAdd(&lcnt[digit], 1u);
+      if (want_p) atomicAdd(&lmass[digit], (unsigned long long)(expf(sl) * 1099511627776.f));
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < bins; b += blockDim.x) {
+      if (lcnt[b]) atomicAdd(&cnt[b], lcnt[b]);
+      if (lmass[b]) atomicAdd(&mass[b], lmass[b]);
+    }
+  } else {
+    for (int v = lo + threadIdx.x; v < hi; v += blockDim.x) {
+      const float sl = (row[v] - top) * inv_t;
+      const uint32_t key = float_key(sl);
+      const uint32_t digit = (key >> fp.shift) & (uint32_t)(bins - 1);
+      const uint32_t high = key >> above;
+      if (want_k && high == prefix_k) atomicAdd(&cnt[digit], 1u);
+      if (want_p && high == prefix_p) atomicAdd(&mass[digit], (unsigned long long)(expf(sl) * 1099511627776.f));
+    }
+  }
+}
+
+template <int PASS>
+__global__ void __launch_bounds__(kWave)
+filter_select_kernel(const float* __restrict__ temperatures, const int* __restrict__ top_ks,
+                     const float* __restrict__ top_ps, unsigned int* __restrict__ hist_cnt,
+                     unsigned long long* __restrict__ hist_mass, unsigned int* __restrict__ state32,
+                     unsigned long long* __restrict__ state64, unsigned int* __restrict__ thresholds, int vocab) {
+  const int r = blockIdx.x;
+  const int lane = threadIdx.x;
+  const int k = top_ks ? top_ks[r] : -1;
+  const float p = top_ps ? top_ps[r] : 1.f;
+  const bool want_k = k > 0 && k < vocab;
+  const bool want_p = p < 1.f;
+  if (!(temperatures[r] > 0.f) || !(want_k || want_p)) {
+    if (PASS == 2 && lane == 0) thresholds[r] = 0u;
+    return;
+  }
+  const FilterPass fp = filter_pass(PASS);
+  const int bins = 1 << fp.width, per = bins / kWave;
+  unsigned int* cnt = hist_cnt + (size_t)r * kDigitBins;
+  unsigned long long* mass = hist_mass + (size_t)r * kDigitBins;
+  // lane l owns bins [per * l, per * l + per): what lies in higher bins, then a walk down its own
+  unsigned int cnt_own = 0u;
+  unsigned long long mass_own = 0ull;
+  for (int b = 0; b < per; ++b) {
+    cnt_own += cnt[per * lane + b];
+    mass_own += mass[per * lane + b];
+  }
+  unsigned int cnt_above = cnt_own;
+  unsigned long long mass_above = mass_own;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {   // inclusive sums over lanes >= this one
+    const unsigned int c = __shfl_down(cnt_above, off, kWave);
+    const unsigned long long m = __shfl_down(mass_above, off, kWave);
+    if (lane + off < kWave) {
+      cnt_above += c;
+      mass_above += m;
+    }
+  }
+  const unsigned long long total_mass = __shfl(mass_above, 0, kWave);
+  cnt_above -= cnt_own;
+  mass_above -= mass_own;
+  const unsigned int prefix_k = PASS ? state32[4 * r] : 0u;
+  const unsigned int prefix_p = PASS ? state32[4 * r + 2] : 0u;
+  const unsigned int need = PASS ? state32[4 * r + 1] : (unsigned int)max(k, 0);
+  const unsigned long long budget = PASS ? state64[r] : (unsigned long long)((double)p * (double)total_mass);
+  unsigned int found_k = 0u, left_k = 0u, found_p = 0u;
+  unsigned long long left_mass = 0ull;
+  bool have_k = false, have_p = false;
+  for (int b = per - 1; b >= 0; --b) {
+    const int bin = per * lane + b;
+    const unsigned int c = cnt[bin];
+    const unsigned long long m = mass[bin];
+    cnt[bin] = 0u;          // the histogram is left empty for the next pass
+    mass[bin] = 0ull;
+    if (want_k && cnt_above < need && cnt_above + c >= need) {   // the k-th largest lies in this bin
+      found_k = prefix_k | ((unsigned int)bin << fp.shift);
+      left_k = need - cnt_above;
+      have_k = true;
+    }
+    // the lowest bin whose higher bins hold no more than the budget
+    if (want_p && mass_above <= budget && (mass_above + m > budget || bin == 0)) {
+      found_p = prefix_p | ((unsigned int)bin << fp.shift);
+      left_mass = budget - mass_above;
+      have_p = true;
+    }
+    cnt_above += c;
+    mass_above += m;
+  }
+  // exactly one lane has found each; lanes write disjoint words
+  if (have_k) {
+    state32[4 * r] = found_k;
+    state32[4 * r + 1] = left_k;
+  }
+  if (have_p) {
+    state32[4 * r + 2] = found_p;
+    state64[r] = left_mass;
+  }
+  if (PASS == 2) {
+    // the larger of the two thresholds; a wave-wide maximum of what the finding lanes hold
+    unsigned int t = max(have_k ? found_k : 0u, have_p ? found_p : 0u);
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) t = max(t, (unsigned int)__shfl_xor((int)t, off, kWave));
+    if (lane == 0) thresholds[r] = t;
+  }
+}
+
 // `ws_vals` / `ws_idx` (rows * 128 elements each, or null) let calls without top-k / top-p spread every row
 // of a large vocabulary over 64 blocks.
+// `ws_filter` (or null): rows * 4096 * 12 + rows * 32 bytes, 8-byte aligned, all zero on entry (it is zero again
+// on return), lets rows with top-k / top-p be spread over 64 blocks too.
 ATOM_EXPORT int atom_sample(const float* logits, const float* temperatures, const int* top_ks, const float* top_ps,
                             const float* noise, long noise_stride, const unsigned long long* seeds,
                             const unsigned long long* counters, int* out, int rows, int vocab, float eps,
-                            float* ws_vals, int* ws_idx, hipStream_t stream) {
+                            float* ws_vals, int* ws_idx, void* ws_filter, hipStream_t stream) {
   if (rows < 0 || vocab <= 0) return ATOM_BAD_SHAPE;
   if (rows == 0) return ATOM_OK;
   static_assert(kArgmaxChunks == kWave, "the pick kernel holds one chunk per lane");
@@ -302,7 +467,8 @@ ATOM_EXPORT int atom_sample(const float* logits, const float* temperatures, cons
       float* race_vals = ws_vals + (size_t)rows * kArgmaxChunks;
       int* race_idx = ws_idx + (size_t)rows * kArgmaxChunks;
       hipLaunchKernelGGL(race_chunks_kernel, dim3(kArgmaxChunks, rows), dim3(256), 0, stream, logits, temperatures,
-                         noise, noise_stride, seeds, counters, ws_vals, ws_idx, race_vals, race_idx, vocab, eps);
+                         noise, noise_stride, seeds, counters, ws_vals, ws_idx, race_vals, race_idx, vocab, eps,
+                         (const unsigned int*)nullptr);
       hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(kWave), 0, stream, race_vals, race_idx, out);
     } else {
       hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(kWave), 0, stream, ws_vals, ws_idx, out);
@@ -310,6 +476,32 @@ ATOM_EXPORT int atom_sample(const float* logits, const float* temperatures, cons
     return launch_status();
   }
   const bool spread = ws_vals && ws_idx && vocab >= 16384 && rows <= 65535;
+  if (spread && ws_filter && temperatures) {
+    // chunk maxima; three rounds of (histogram over 64 blocks a row, a walk by one wave a row); the race
+    // among the kept tokens of each chunk; the pick among the chunks' winners
+    unsigned long long* hist_mass = (unsigned long long*)ws_filter;
+    unsigned long long* state64 = hist_mass + (size_t)rows * kDigitBins;
+    unsigned int* hist_cnt = (unsigned int*)(state64 + rows);
+    unsigned int* state32 = hist_cnt + (size_t)rows * kDigitBins;
+    unsigned int* thresholds = state32 + (size_t)rows * 4;   // 4 + 1 words a row: rows * 32 bytes hold them
+    const dim3 wide(kArgmaxChunks, rows);
+    hipLaunchKernelGGL(argmax_chunks_kernel, wide, dim3(256), 0, stream, logits, ws_vals, ws_idx, vocab);
+#define FILTER_ROUND(P)                                                                                            \
+  hipLaunchKernelGGL((filter_hist_kernel<P>), wide, dim3(256), 0, stream, logits, temperatures, top_ks, top_ps,    \
+                     ws_vals, hist_cnt, hist_mass, state32, vocab);                                                \
+  hipLaunchKernelGGL((filter_select_kernel<P>), dim3(rows), dim3(kWave), 0, stream, temperatures, top_ks, top_ps,  \
+                     hist_cnt, hist_mass, state32, state64, thresholds, vocab)
+    FILTER_ROUND(0);
+    FILTER_ROUND(1);
+    FILTER_ROUND(2);
+#undef FILTER_ROUND
+    float* race_vals = ws_vals + (size_t)rows * kArgmaxChunks;
+    int* race_idx = ws_idx + (size_t)rows * kArgmaxChunks;
+    hipLaunchKernelGGL(race_chunks_kernel, wide, dim3(256), 0, stream, logits, temperatures, noise, noise_stride,
+                       seeds, counters, ws_vals, ws_idx, race_vals, race_idx, vocab, eps, thresholds);
+    hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(kWave), 0, stream, race_vals, race_idx, out);
+    return launch_status();
+  }
   if (spread)   // the rows' maxima by 64 blocks a row instead of one
     hipLaunchKernelGGL(argmax_chunks_kernel, dim3(kArgmaxChunks, rows), dim3(256), 0, stream, logits, ws_vals, ws_idx,
                        vocab);

@@ -125,6 +125,7 @@ class HipKernels:
         self.use_mfma_attention = True
         self.use_tiled_prefill = True
         self._ws: dict[str, torch.Tensor] = {}
+        self._zeroed: dict[str, torch.Tensor] = {}   # workspaces that every kernel leaves all zero
         self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
 
     def workspace(self, name: str, numel: int, dtype=torch.float32) -> torch.Tensor:
@@ -480,10 +481,19 @@ class HipKernels:
         # every row's maximum (and, without filters, its race) is spread over 64 blocks: chunk maxima, chunk winners
         ws_vals = self.workspace("sample_vals", rows * 128)
         ws_idx = self.workspace("sample_idx", rows * 128, torch.int32)
+        ws_filter = None
+        if temperatures is not None and (top_ks is not None or top_ps is not None) and vocab >= 16384:
+            # histograms of the threshold search: zero when made, and left zero by every call
+            need = rows * (4096 * 12 + 32)
+            ws_filter = self._zeroed.get("sample_filter")
+            if ws_filter is None or ws_filter.numel() < need or torch.cuda.is_current_stream_capturing():
+                ws_filter = torch.zeros(need, dtype=torch.uint8, device=self.device)
+                if not torch.cuda.is_current_stream_capturing():
+                    self._zeroed["sample_filter"] = ws_filter
         self._done("sample", self.lib.atom_sample(
             _ptr(logits), _ptr(temperatures), _ptr(top_ks), _ptr(top_ps), _ptr(noise), ctypes.c_long(stride),
             _ptr(seeds), _ptr(counters), _ptr(out), rows, vocab, ctypes.c_float(eps), _ptr(ws_vals), _ptr(ws_idx),
-            self._stream()))
+            _ptr(ws_filter), self._stream()))
         return out
 
     def exponential_noise(self, seeds, counters, vocab: int):

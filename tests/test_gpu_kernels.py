@@ -430,6 +430,25 @@ def test_sample_at_a_real_vocabulary(top_k, top_p):
     assert out.cpu().tolist() == want.tolist()
 
 
+def test_sample_rows_with_different_filters_at_a_real_vocabulary():
+    """Rows of one call with their own temperature, top-k and top-p (off, 1, larger than the vocabulary, a p that
+    keeps the likeliest token only, greedy rows between); called three times, because the kernels' histograms
+    must be left empty for the next call."""
+    rows, vocab = 7, 151936
+    temps = torch.tensor([0.7, 1.0, 0.0, 1.3, 0.6, 0.9, 0.0], dtype=torch.float32)
+    ks = torch.tensor([-1, 1, 50, 200000, 7, -1, -1], dtype=torch.int32)
+    ps = torch.tensor([0.5, 1.0, 0.4, 0.9, 1.0, 1e-4, 0.3], dtype=torch.float32)
+    for call in range(3):
+        logits = rnd((rows, vocab), torch.float32, 50 + call, 2.0 + call)
+        noise = torch.empty((rows, vocab)).exponential_(generator=torch.Generator().manual_seed(60 + call))
+        out = torch.empty(rows, dtype=torch.int32, device=DEV)
+        gpu_ops().sample(logits.to(DEV), temps.to(DEV), out, top_ks=ks.to(DEV), top_ps=ps.to(DEV), noise=noise.to(DEV))
+        want = torch.empty(rows, dtype=torch.int32)
+        PLAIN.sample(logits, temps, want, top_ks=ks, top_ps=ps, noise=noise)
+        assert out.cpu().tolist() == want.tolist(), call
+        assert int(out[1]) == int(logits[1].argmax()) and int(out[5]) == int(logits[5].argmax())
+
+
 def test_sample_frequencies_follow_softmax():
     vocab, draws = 11, 20000
     logits = torch.tensor([[2.0, 1.0, 0.5, 0.0, -1.0, 1.5, 0.2, -3.0, 0.9, 1.1, -0.5]])
