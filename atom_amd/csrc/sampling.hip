@@ -1,4 +1,5 @@
-// Sampling from float32 logits, one block per row.
+// Sampling from float32 logits: one block per row, or, for large vocabularies (from 16,384 tokens, given
+// workspaces), every row spread over 64 blocks (chunk maxima, threshold rounds, the race per chunk, a pick).
 //
 //   greedy (temperature 0):  lowest index of the maximum.
 //   otherwise:               token = argmax_v softmax(logits / T)_v / (E_v + eps),  E_v ~ Exp(1),
