@@ -50,6 +50,8 @@ class EngineArgs:
     torch_profiler_dir: str | None = None
     mark_trace: bool = False
     deferred_output: bool = True
+    level: int = 3
+    cudagraph_mode: str = "FULL"
     hf_overrides: dict | None = None
     num_kvcache_blocks: int = -1
     dtype: str = "bf16"
@@ -82,6 +84,13 @@ class EngineArgs:
                             help="Name every operation's kernels in profiler traces (record_function spans).")
         parser.add_argument("--deferred-output", action=argparse.BooleanOptionalAction, default=True,
                             help="Launch the next decode step before the host has read the last one's tokens.")
+        # the reference's two switches of its tracing compiler and graph modes (atom/model_engine/arg_utils.py
+        # :195-208): there is no compiler here, so the level changes nothing; NONE means --enforce-eager, every
+        # other mode the one kind of graph this engine has (a whole decode step)
+        parser.add_argument("--level", type=int, default=3, help="Accepted for the reference's command lines; no effect.")
+        parser.add_argument("--cudagraph-mode", type=str, default="FULL",
+                            choices=["NONE", "PIECEWISE", "FULL", "FULL_AND_PIECEWISE", "AF_PIECEWISE"],
+                            help="NONE: never replay graphs (as --enforce-eager); any other: whole decode steps.")
         parser.add_argument("--hf-overrides", type=json.loads, default=None, help="JSON dict of config.json overrides.")
         parser.add_argument("--num-kvcache-blocks", type=int, default=-1, help="Cache pages (-1: from free memory).")
         parser.add_argument("--dtype", choices=["bf16", "bfloat16", "fp32", "float32"], default="bf16",
@@ -98,6 +107,9 @@ class EngineArgs:
         kwargs = {f.name: getattr(self, f.name) for f in fields(self) if f.name != "model"}
         kwargs["kv_cache_block_size"] = kwargs.pop("block_size")
         kwargs["cudagraph_capture_sizes"] = parse_size_list(kwargs["cudagraph_capture_sizes"])
+        kwargs.pop("level")
+        if kwargs.pop("cudagraph_mode") == "NONE":
+            kwargs["enforce_eager"] = True
         return kwargs
 
     def create_engine(self, tokenizer=None):

@@ -115,6 +115,9 @@ def test_cli_flags_in_both_spellings():
                                                     "--mark-trace"]))
     assert (a.model, a.max_model_len, a.block_size, a.enable_chunked_prefill, a.max_num_seqs) == ("m", 99, 32, False, 7)
     assert a.mark_trace and not EngineArgs(model="m").mark_trace
+    b = EngineArgs.from_cli_args(parser.parse_args(["--model", "m", "--level", "0", "--cudagraph-mode", "NONE"]))
+    assert b._get_engine_kwargs()["enforce_eager"] and "level" not in b._get_engine_kwargs()
+    assert not a._get_engine_kwargs()["enforce_eager"]
     kw = a._get_engine_kwargs()
     assert kw["kv_cache_block_size"] == 32 and "block_size" not in kw
     assert kw["cudagraph_capture_sizes"][:3] == [1, 2, 4]
