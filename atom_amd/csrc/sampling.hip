@@ -313,7 +313,7 @@ filter_hist_kernel(const float* __restrict__ logits, const float* __restrict__ t
                    const float* __restrict__ max_vals, unsigned int* __restrict__ hist_cnt,
                    unsigned long long* __restrict__ hist_mass, const unsigned int* __restrict__ state32, int vocab) {
   const int r = blockIdx.y;
-  const int chunk = blockIdx.x;
+  const int chunk = blockIdx.x;          // of gridDim.x chunks of the row (its own division, not the maxima's)
   const float temp = temperatures[r];
   const int k = top_ks ? top_ks[r] : -1;
   const bool want_k = k > 0 && k < vocab;
@@ -326,7 +326,7 @@ filter_hist_kernel(const float* __restrict__ logits, const float* __restrict__ t
   const int bins = 1 << fp.width, above = fp.shift + fp.width;
   const uint32_t prefix_k = PASS ? state32[4 * r] >> above : 0u;
   const uint32_t prefix_p = PASS ? state32[4 * r + 2] >> above : 0u;
-  const int per = (vocab + kArgmaxChunks - 1) / kArgmaxChunks;
+  const int per = (vocab + (int)gridDim.x - 1) / (int)gridDim.x;
   const int lo = chunk * per, hi = min(vocab, lo + per);
   const float* row = logits + (size_t)r * vocab;
   const float inv_t = 1.f / temp;
@@ -364,89 +364,103 @@ filter_hist_kernel(const float* __restrict__ logits, const float* __restrict__ t
   }
 }
 
+constexpr int kSelectThreads = 256;
+
 template <int PASS>
-__global__ void __launch_bounds__(kWave)
+__global__ void __launch_bounds__(kSelectThreads)
 filter_select_kernel(const float* __restrict__ temperatures, const int* __restrict__ top_ks,
                      const float* __restrict__ top_ps, unsigned int* __restrict__ hist_cnt,
                      unsigned long long* __restrict__ hist_mass, unsigned int* __restrict__ state32,
                      unsigned long long* __restrict__ state64, unsigned int* __restrict__ thresholds, int vocab) {
+  __shared__ unsigned int tot_cnt[kSelectThreads / kWave];
+  __shared__ unsigned long long tot_mass[kSelectThreads / kWave];
+  __shared__ unsigned int result[2];   // the digits of u_k and u_p found in this pass
   const int r = blockIdx.x;
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x;
   const int k = top_ks ? top_ks[r] : -1;
   const float p = top_ps ? top_ps[r] : 1.f;
   const bool want_k = k > 0 && k < vocab;
   const bool want_p = p < 1.f;
   if (!(temperatures[r] > 0.f) || !(want_k || want_p)) {
-    if (PASS == 2 && lane == 0) thresholds[r] = 0u;
+    if (PASS == 2 && tid == 0) thresholds[r] = 0u;
     return;
   }
   const FilterPass fp = filter_pass(PASS);
-  const int bins = 1 << fp.width, per = bins / kWave;
+  constexpr int BINS = PASS == 2 ? 256 : kDigitBins;
+  constexpr int PER = BINS / kSelectThreads;   // thread t owns bins [PER * t, PER * t + PER)
   unsigned int* cnt = hist_cnt + (size_t)r * kDigitBins;
   unsigned long long* mass = hist_mass + (size_t)r * kDigitBins;
-  // lane l owns bins [per * l, per * l + per): what lies in higher bins, then a walk down its own
+  unsigned int c[PER];
+  unsigned long long m[PER];
   unsigned int cnt_own = 0u;
   unsigned long long mass_own = 0ull;
-  for (int b = 0; b < per; ++b) {
-    cnt_own += cnt[per * lane + b];
-    mass_own += mass[per * lane + b];
+#pragma unroll
+  for (int b = 0; b < PER; ++b) {
+    c[b] = cnt[PER * tid + b];
+    m[b] = mass[PER * tid + b];
+    cnt[PER * tid + b] = 0u;          // the histogram is left empty for the next pass
+    mass[PER * tid + b] = 0ull;
+    cnt_own += c[b];
+    mass_own += m[b];
   }
+  // what lies in the bins above this thread's, and the row's total mass: sums over the higher lanes of the
+  // wave by shuffles, over the higher waves through LDS
+  const int lane = tid & (kWave - 1), wave = tid / kWave;
   unsigned int cnt_above = cnt_own;
   unsigned long long mass_above = mass_own;
 #pragma unroll
   for (int off = 1; off < kWave; off <<= 1) {   // inclusive sums over lanes >= this one
-    const unsigned int c = __shfl_down(cnt_above, off, kWave);
-    const unsigned long long m = __shfl_down(mass_above, off, kWave);
+    const unsigned int cc = __shfl_down(cnt_above, off, kWave);
+    const unsigned long long mm = __shfl_down(mass_above, off, kWave);
     if (lane + off < kWave) {
-      cnt_above += c;
-      mass_above += m;
+      cnt_above += cc;
+      mass_above += mm;
     }
   }
-  const unsigned long long total_mass = __shfl(mass_above, 0, kWave);
+  if (lane == 0) {
+    tot_cnt[wave] = cnt_above;
+    tot_mass[wave] = mass_above;
+  }
+  if (tid < 2) result[tid] = 0u;
+  __syncthreads();
   cnt_above -= cnt_own;
   mass_above -= mass_own;
+  unsigned long long total_mass = 0ull;
+#pragma unroll
+  for (int w = 0; w < kSelectThreads / kWave; ++w) {
+    total_mass += tot_mass[w];
+    if (w > wave) {
+      cnt_above += tot_cnt[w];
+      mass_above += tot_mass[w];
+    }
+  }
   const unsigned int prefix_k = PASS ? state32[4 * r] : 0u;
   const unsigned int prefix_p = PASS ? state32[4 * r + 2] : 0u;
   const unsigned int need = PASS ? state32[4 * r + 1] : (unsigned int)max(k, 0);
   const unsigned long long budget = PASS ? state64[r] : (unsigned long long)((double)p * (double)total_mass);
-  unsigned int found_k = 0u, left_k = 0u, found_p = 0u;
-  unsigned long long left_mass = 0ull;
-  bool have_k = false, have_p = false;
-  for (int b = per - 1; b >= 0; --b) {
-    const int bin = per * lane + b;
-    const unsigned int c = cnt[bin];
-    const unsigned long long m = mass[bin];
-    cnt[bin] = 0u;          // the histogram is left empty for the next pass
-    mass[bin] = 0ull;
-    if (want_k && cnt_above < need && cnt_above + c >= need) {   // the k-th largest lies in this bin
-      found_k = prefix_k | ((unsigned int)bin << fp.shift);
-      left_k = need - cnt_above;
-      have_k = true;
+  __syncthreads();   // every thread has read the state before the finders write it
+#pragma unroll
+  for (int b = PER - 1; b >= 0; --b) {
+    const int bin = PER * tid + b;
+    if (want_k && cnt_above < need && cnt_above + c[b] >= need) {   // the k-th largest lies in this bin
+      const unsigned int found = prefix_k | ((unsigned int)bin << fp.shift);
+      state32[4 * r] = found;
+      state32[4 * r + 1] = need - cnt_above;
+      result[0] = found;
     }
     // the lowest bin whose higher bins hold no more than the budget
-    if (want_p && mass_above <= budget && (mass_above + m > budget || bin == 0)) {
-      found_p = prefix_p | ((unsigned int)bin << fp.shift);
-      left_mass = budget - mass_above;
-      have_p = true;
+    if (want_p && mass_above <= budget && (mass_above + m[b] > budget || bin == 0)) {
+      const unsigned int found = prefix_p | ((unsigned int)bin << fp.shift);
+      state32[4 * r + 2] = found;
+      state64[r] = budget - mass_above;
+      result[1] = found;
     }
-    cnt_above += c;
-    mass_above += m;
-  }
-  // exactly one lane has found each; lanes write disjoint words
-  if (have_k) {
-    state32[4 * r] = found_k;
-    state32[4 * r + 1] = left_k;
-  }
-  if (have_p) {
-    state32[4 * r + 2] = found_p;
-    state64[r] = left_mass;
+    cnt_above += c[b];
+    mass_above += m[b];
   }
   if (PASS == 2) {
-    // the larger of the two thresholds; a wave-wide maximum of what the finding lanes hold
-    unsigned int t = max(have_k ? found_k : 0u, have_p ? found_p : 0u);
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) t = max(t, (unsigned int)__shfl_xor((int)t, off, kWave));
-    if (lane == 0) thresholds[r] = t;
+    __syncthreads();
+    if (tid == 0) thresholds[r] = max(result[0], result[1]);   // the race keeps keys >= both thresholds
   }
 }
 
@@ -486,11 +500,14 @@ ATOM_EXPORT int atom_sample(const float* logits, const float* temperatures, cons
     unsigned int* state32 = hist_cnt + (size_t)rows * kDigitBins;
     unsigned int* thresholds = state32 + (size_t)rows * 4;   // 4 + 1 words a row: rows * 32 bytes hold them
     const dim3 wide(kArgmaxChunks, rows);
+    const dim3 hist_grid = wide;
     hipLaunchKernelGGL(argmax_chunks_kernel, wide, dim3(256), 0, stream, logits, ws_vals, ws_idx, vocab);
 #define FILTER_ROUND(P)                                                                                            \
-  hipLaunchKernelGGL((filter_hist_kernel<P>), wide, dim3(256), 0, stream, logits, temperatures, top_ks, top_ps,    \
+  hipLaunchKernelGGL((filter_hist_kernel<P>), hist_grid, dim3(256), 0, stream, logits, temperatures, top_ks,       \
+                     top_ps,                                                                                      \
                      ws_vals, hist_cnt, hist_mass, state32, vocab);                                                \
-  hipLaunchKernelGGL((filter_select_kernel<P>), dim3(rows), dim3(kWave), 0, stream, temperatures, top_ks, top_ps,  \
+  hipLaunchKernelGGL((filter_select_kernel<P>), dim3(rows), dim3(kSelectThreads), 0, stream, temperatures, top_ks, \
+                     top_ps,                                                                                      \
                      hist_cnt, hist_mass, state32, state64, thresholds, vocab)
     FILTER_ROUND(0);
     FILTER_ROUND(1);
