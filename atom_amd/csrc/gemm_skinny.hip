@@ -210,6 +210,188 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
   }
 }
 
+// ---- 17 to 64 rows of x.  With that many rows a useful slice of x no longer fits beside the weights'
+// layout-change areas, and the block's K range is long, so x is streamed like the weights: a chunk is
+// 128 k of the block's 64 rows of w and of the rows of x, each wave loads 16 rows of either (the same
+// whole-cache-line loads as above, four chunks in flight a wave) and writes them to one of two LDS
+// buffers; after the block's barrier every wave multiplies the 64 rows of w with its own 16 rows of x.
+// A block owns 64 rows of w and a range of K; products with many rows of w are not cut.
+constexpr int kMidRows = 128;               // rows of a chunk in LDS: 64 of w, then up to 64 of x
+constexpr int kMidBuf = kMidRows * kARow;   // LDS bytes of a chunk
+constexpr int kMidSlice = 1024;             // K is cut in multiples of this
+
+template <bool GATE>
+__global__ void __launch_bounds__(256, 2) gemm_mid_kernel(SkinnyParams p) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];   // two chunks
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;          // loads rows 16 wave .. 16 wave + 15 of w and of x; multiplies with those of x
+  const int r16 = lane & 15;
+  const int g = lane >> 4;
+  const int k = p.k;
+  const int tile = blockIdx.x / p.splits;
+  const int split = blockIdx.x - tile * p.splits;
+  const int k_begin = split * p.kslice;
+  const int k_end = min(k, k_begin + p.kslice);
+  const int total = (k_end - k_begin + 127) / 128;   // chunks
+
+  auto w_row = [&](int j) -> int {
+    if (GATE) {
+      const int col = tile * 32 + (wave & 1) * 16 + j;
+      return min(col, p.inter - 1) + (wave >= 2 ? p.inter : 0);
+    }
+    return min(tile * kSkinnyRows + wave * 16 + j, p.n - 1);
+  };
+  const bool active = 16 * wave < p.m;
+  const bf16_t* wrow[4];
+  const bf16_t* xrow[4];
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg) {
+    wrow[rg] = p.w + (size_t)w_row(4 * rg + g) * k + 8 * r16;
+    xrow[rg] = p.x + (size_t)min(16 * wave + 4 * rg + g, p.m - 1) * k + 8 * r16;
+  }
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  f32x4 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 a[16], xa[16];
+  // chunk `ci` into the registers of `slot`: this lane's 16 bytes of four rows of w and of x
+  auto load_chunk = [&](int slot, int ci) {
+    const int kk = k_begin + 128 * ci;
+    const bool in = kk + 8 * r16 < k_end;
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg)
+      a[4 * slot + rg] = in ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[rg] + kk)) : zero;
+    if (active) {
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg)
+        xa[4 * slot + rg] = in ? *reinterpret_cast<const bf16x8*>(xrow[rg] + kk) : zero;
+    }
+  };
+#pragma unroll
+  for (int slot = 0; slot < 4; ++slot)
+    if (slot < total) load_chunk(slot, slot);
+
+  for (int base = 0; base < total; base += 4) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int ci = base + c;
+      if (ci < total) {   // the same in every wave of the block
+        char* buf = lds + (c & 1) * kMidBuf;
+        // the two buffers take turns: a wave that writes chunk ci has passed the barrier of chunk ci - 1,
+        // which every wave reaches only after it has read chunk ci - 2
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg)
+          *reinterpret_cast<bf16x8*>(buf + (16 * wave + 4 * rg + g) * kARow + r16 * 16) = a[4 * c + rg];
+        if (active) {
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg)
+            *reinterpret_cast<bf16x8*>(buf + (64 + 16 * wave + 4 * rg + g) * kARow + r16 * 16) = xa[4 * c + rg];
+        }
+        if (ci + 4 < total) load_chunk(c, ci + 4);
+        __syncthreads();
+        if (active) {
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const bf16x8 bv = *reinterpret_cast<const bf16x8*>(buf + (64 + 16 * wave + r16) * kARow + u * 64 + g * 16);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const bf16x8 av = *reinterpret_cast<const bf16x8*>(buf + (16 * j + r16) * kARow + u * 64 + g * 16);
+              acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc[j], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+  }
+
+  // lane (r16, g) holds, for row m = 16 wave + r16 of x, columns 16 j + 4 g .. + 3 of the block's 64
+  const int m = 16 * wave + r16;
+  if (!active || m >= p.m) return;
+  const bool vec = (p.n & 3) == 0 && (!GATE || (p.inter & 3) == 0);
+  if (p.splits > 1) {
+    float* out_row = p.partial + ((size_t)split * p.m + m) * p.n;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = 16 * j + 4 * g;
+      int col, limit;
+      if (GATE) {
+        col = tile * 32 + (c & 31) + (c >= 32 ? p.inter : 0);
+        limit = (c >= 32 ? 2 : 1) * p.inter;
+      } else {
+        col = tile * kSkinnyRows + c;
+        limit = p.n;
+      }
+      if (vec) {
+        if (col < limit) *reinterpret_cast<f32x4*>(out_row + col) = acc[j];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (col + i < limit) out_row[col + i] = acc[j][i];
+      }
+    }
+    return;
+  }
+  if (GATE) {
+    bf16_t* out_row = reinterpret_cast<bf16_t*>(p.y) + (size_t)m * p.inter;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = tile * 32 + 16 * j + 4 * g;
+      bf16_t r[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float gv = acc[j][i], uv = acc[j + 2][i];
+        if (p.bias && col + i < p.inter) {
+          gv += p.bias[col + i];
+          uv += p.bias[p.inter + col + i];
+        }
+        r[i] = from_f32<bf16_t>(gv / (1.f + expf(-gv)) * uv);
+      }
+      if (vec) {
+        if (col < p.inter) *reinterpret_cast<uint2*>(out_row + col) = *reinterpret_cast<const uint2*>(r);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (col + i < p.inter) out_row[col + i] = r[i];
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int col = tile * kSkinnyRows + 16 * j + 4 * g;
+    f32x4 v = acc[j];
+    if (p.bias) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (col + i < p.n) v[i] += p.bias[col + i];
+    }
+    if (p.out_f32) {
+      float* out_row = reinterpret_cast<float*>(p.y) + (size_t)m * p.n;
+      if (vec) {
+        if (col < p.n) *reinterpret_cast<f32x4*>(out_row + col) = v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (col + i < p.n) out_row[col + i] = v[i];
+      }
+    } else {
+      bf16_t* out_row = reinterpret_cast<bf16_t*>(p.y) + (size_t)m * p.n;
+      bf16_t r[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) r[i] = from_f32<bf16_t>(v[i]);
+      if (vec) {
+        if (col < p.n) *reinterpret_cast<uint2*>(out_row + col) = *reinterpret_cast<const uint2*>(r);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (col + i < p.n) out_row[col + i] = r[i];
+      }
+    }
+  }
+}
+
 // y[m, n] = sum over splits of partial[s][m][n] (+ bias), in slice order.
 template <typename TY>
 __global__ void splitk_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ bias,
@@ -241,6 +423,22 @@ static SkinnyPlan skinny_plan(int m, int tiles, int k) {
   return plan;
 }
 
+// More than 16 rows: K is cut only as far as it takes to have about 256 blocks, in slices that are a
+// multiple of the 1024 k a wave holds of x.
+static SkinnyPlan mid_plan(int tiles, int k) {
+  SkinnyPlan plan{};
+  const int units = (k + kMidSlice - 1) / kMidSlice;
+  int s = tiles >= 192 ? 1 : (320 + tiles - 1) / tiles;
+  s = max(1, min(s, units));
+  const int per = (units + s - 1) / s;
+  plan.kslice = per * kMidSlice;
+  plan.splits = (units + per - 1) / per;
+  plan.xk = 0;
+  return plan;
+}
+
+static SkinnyPlan plan_for(int m, int tiles, int k) { return m > 16 ? mid_plan(tiles, k) : skinny_plan(m, tiles, k); }
+
 // 1 if the skinny kernel takes this product.
 ATOM_EXPORT int atom_gemm_skinny_supports(int m, int n, int k) {
   return m >= 1 && m <= 64 && n >= 1 && k >= 8 && k % 8 == 0;
@@ -248,7 +446,7 @@ ATOM_EXPORT int atom_gemm_skinny_supports(int m, int n, int k) {
 
 // Into how many slices atom_gemm_skinny cuts K for this product (1: it writes y itself).
 ATOM_EXPORT int atom_gemm_skinny_splits(int m, int n, int k, int gate) {
-  return skinny_plan(max(m, 1), skinny_tiles(n, gate), k).splits;
+  return plan_for(max(m, 1), skinny_tiles(n, gate), k).splits;
 }
 
 // gate == 0: x w^T, n columns.  gate == 1: w is [2 n, k] (n gate rows, then n up rows).
@@ -268,11 +466,30 @@ ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias
   p.n = gate ? 2 * n : n;
   p.inter = gate ? n : 0;
   p.tiles = skinny_tiles(n, gate);
-  const SkinnyPlan plan = skinny_plan(m, p.tiles, k);
+  const SkinnyPlan plan = plan_for(m, p.tiles, k);
   p.splits = plan.splits; p.kslice = plan.kslice; p.xk = plan.xk;
   if (p.splits > 1 ? partial == nullptr : y == nullptr) return ATOM_BAD_SHAPE;
   const long blocks = (long)p.tiles * p.splits;
   if (blocks > 0x7fffffffL) return ATOM_TOO_LARGE;
+  if (m > 16) {
+    if ((uintptr_t)y & 15) return ATOM_BAD_SHAPE;
+    // two chunks of LDS are more than a launch gets by default: allow it once per kernel
+#define GO_MID(G)                                                                                          \
+  do {                                                                                                     \
+    static bool allowed = false;                                                                           \
+    if (!allowed) {                                                                                        \
+      if (hipFuncSetAttribute((const void*)gemm_mid_kernel<G>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                              2 * kMidBuf) != hipSuccess)                                                  \
+        return ATOM_LAUNCH_FAILED;                                                                         \
+      allowed = true;                                                                                      \
+    }                                                                                                      \
+    hipLaunchKernelGGL(gemm_mid_kernel<G>, dim3(blocks), dim3(256), 2 * kMidBuf, stream, p);               \
+  } while (0)
+    if (gate) GO_MID(true);
+    else GO_MID(false);
+#undef GO_MID
+    return launch_status();
+  }
   const size_t lds = (size_t)4 * kAWave + max((size_t)m * (p.xk * 2 + 16), (size_t)m * (kSkinnyRows + 1) * 4);
   const int mt = (m + 15) / 16;
   // 64 rows of x need a little more LDS than a launch gets by default: allow it once per kernel

@@ -121,7 +121,7 @@ class HipKernels:
         # bfloat16 products of few rows run this library's own weight-streaming kernel.  It takes up to 64
         # rows; beyond 16 (one matrix-core tile of rows) the BLAS library's kernels are faster on gfx950.
         self.use_skinny_gemm = True
-        self.skinny_max_rows = 16
+        self.skinny_max_rows = 64
         self.use_mfma_attention = True
         self.use_tiled_prefill = True
         self._ws: dict[str, torch.Tensor] = {}
