@@ -2,6 +2,7 @@
 // float32 accumulation on the matrix cores.  This is the decode-step product: the
 // weight matrix is streamed from memory once and the work is bound by that stream.
 //
+// Up to 16 rows of x (gemm_skinny_kernel; 17 to 64 rows: gemm_mid_kernel, described at its place).
 // A block of four waves owns 64 rows of w (64 output columns) and a slice of K; each
 // wave owns 16 of the rows and walks its part of the slice in shots of 512 k.  For a shot
 // a wave issues all its 16 loads at once, non-temporal, each covering 256 contiguous
@@ -17,7 +18,7 @@
 // block writes its partial tile to partial[split][m][n] (float32).  Whoever reads the
 // product next adds the slices in slice order: the norm, the rotation kernel, SiLU-mul,
 // or atom_splitk_reduce.  The sum has one fixed order, so a row's result does not
-// depend on its batch.
+// depend on the rows beside it (to the bit within one of the two kernels; they cut K differently).
 //
 // Epilogues when K is not cut: plain (bias optional, bfloat16 or float32 out), or
 // SiLU-gate: w holds `inter` gate rows then `inter` up rows, a block owns 32 columns of
@@ -210,22 +211,26 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
   }
 }
 
-// ---- 17 to 64 rows of x.  With that many rows a useful slice of x no longer fits beside the weights'
-// layout-change areas, and the block's K range is long, so x is streamed like the weights: a chunk is
-// 128 k of the block's 64 rows of w and of the rows of x, each wave loads 16 rows of either (the same
-// whole-cache-line loads as above, four chunks in flight a wave) and writes them to one of two LDS
-// buffers; after the block's barrier every wave multiplies the 64 rows of w with its own 16 rows of x.
-// A block owns 64 rows of w and a range of K; products with many rows of w are not cut.
-constexpr int kMidRows = 128;               // rows of a chunk in LDS: 64 of w, then up to 64 of x
-constexpr int kMidBuf = kMidRows * kARow;   // LDS bytes of a chunk
-constexpr int kMidSlice = 1024;             // K is cut in multiples of this
+// ---- 17 to 64 rows of x.  With that many rows a useful slice of x no longer fits in LDS beside the
+// weights' layout-change areas, so x is streamed like the weights.  A block of W waves (4 to 8) owns
+// 16 W rows of w and a range of K; a chunk is 128 k of those rows and of the rows of x.  Each wave loads
+// its own 16 rows of w and a share of the rows of x (the same whole-cache-line loads as above, four
+// chunks in flight a wave) and writes them to one of two LDS buffers; after the block's barrier it
+// multiplies its rows of w with every 16 rows of x.  The more waves, the fewer times x is read; wide
+// products take the W that fills the chip best and are not cut, narrow ones four waves and as many
+// slices of K as it takes to have about 256 blocks.
+//
+// SiLU-gate: a wave's 16 rows are 8 gate and 8 up rows of the same 8 columns, ordered so that a lane's
+// four results are two gate values and the two up values of the same columns.
+constexpr int kMidSlice = 1024;   // K is cut in multiples of this
 
-template <bool GATE>
-__global__ void __launch_bounds__(256, 2) gemm_mid_kernel(SkinnyParams p) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];   // two chunks
+template <int MT, bool GATE>
+__global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];   // two chunks of 16 W + 16 MT rows
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
-  const int wave = tid / kWave;          // loads rows 16 wave .. 16 wave + 15 of w and of x; multiplies with those of x
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int waves = blockDim.x / kWave;
   const int r16 = lane & 15;
   const int g = lane >> 4;
   const int k = p.k;
@@ -234,40 +239,42 @@ __global__ void __launch_bounds__(256, 2) gemm_mid_kernel(SkinnyParams p) {
   const int k_begin = split * p.kslice;
   const int k_end = min(k, k_begin + p.kslice);
   const int total = (k_end - k_begin + 127) / 128;   // chunks
+  const int chunk_bytes = (16 * waves + 16 * MT) * kARow;
 
+  // first column of this wave; row j (0..15) of the wave in w
+  const int col0 = GATE ? (tile * waves + wave) * 8 : (tile * waves + wave) * 16;
   auto w_row = [&](int j) -> int {
-    if (GATE) {
-      const int col = tile * 32 + (wave & 1) * 16 + j;
-      return min(col, p.inter - 1) + (wave >= 2 ? p.inter : 0);
-    }
-    return min(tile * kSkinnyRows + wave * 16 + j, p.n - 1);
+    if (GATE) return min(col0 + 2 * (j >> 2) + (j & 1), p.inter - 1) + ((j & 2) ? p.inter : 0);
+    return min(col0 + j, p.n - 1);
   };
-  const bool active = 16 * wave < p.m;
+  // load (rg) of a chunk of w: this lane's 16 bytes of row 4 rg + g;  load (q) of x: of row 4 (wave + waves q) + g
   const bf16_t* wrow[4];
   const bf16_t* xrow[4];
+  int xat[4];
+  bool xmine[4];   // the same in all lanes of a wave
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg) {
     wrow[rg] = p.w + (size_t)w_row(4 * rg + g) * k + 8 * r16;
-    xrow[rg] = p.x + (size_t)min(16 * wave + 4 * rg + g, p.m - 1) * k + 8 * r16;
+    const int four = wave + waves * rg;   // which four rows of x
+    xmine[rg] = four < 4 * MT;
+    xat[rg] = (16 * waves + 4 * four + g) * kARow + r16 * 16;
+    xrow[rg] = p.x + (size_t)min(4 * four + g, p.m - 1) * k + 8 * r16;
   }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  f32x4 acc[4];
+  f32x4 acc[MT];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   bf16x8 a[16], xa[16];
-  // chunk `ci` into the registers of `slot`: this lane's 16 bytes of four rows of w and of x
   auto load_chunk = [&](int slot, int ci) {
     const int kk = k_begin + 128 * ci;
     const bool in = kk + 8 * r16 < k_end;
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg)
       a[4 * slot + rg] = in ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[rg] + kk)) : zero;
-    if (active) {
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg)
-        xa[4 * slot + rg] = in ? *reinterpret_cast<const bf16x8*>(xrow[rg] + kk) : zero;
-    }
+    for (int rg = 0; rg < 4; ++rg)
+      if (xmine[rg]) xa[4 * slot + rg] = in ? *reinterpret_cast<const bf16x8*>(xrow[rg] + kk) : zero;
   };
 #pragma unroll
   for (int slot = 0; slot < 4; ++slot)
@@ -278,90 +285,91 @@ __global__ void __launch_bounds__(256, 2) gemm_mid_kernel(SkinnyParams p) {
     for (int c = 0; c < 4; ++c) {
       const int ci = base + c;
       if (ci < total) {   // the same in every wave of the block
-        char* buf = lds + (c & 1) * kMidBuf;
+        char* buf = lds + (c & 1) * chunk_bytes;
         // the two buffers take turns: a wave that writes chunk ci has passed the barrier of chunk ci - 1,
         // which every wave reaches only after it has read chunk ci - 2
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg)
           *reinterpret_cast<bf16x8*>(buf + (16 * wave + 4 * rg + g) * kARow + r16 * 16) = a[4 * c + rg];
-        if (active) {
 #pragma unroll
-          for (int rg = 0; rg < 4; ++rg)
-            *reinterpret_cast<bf16x8*>(buf + (64 + 16 * wave + 4 * rg + g) * kARow + r16 * 16) = xa[4 * c + rg];
-        }
+        for (int rg = 0; rg < 4; ++rg)
+          if (xmine[rg]) *reinterpret_cast<bf16x8*>(buf + xat[rg]) = xa[4 * c + rg];
         if (ci + 4 < total) load_chunk(c, ci + 4);
         __syncthreads();
-        if (active) {
 #pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const bf16x8 bv = *reinterpret_cast<const bf16x8*>(buf + (64 + 16 * wave + r16) * kARow + u * 64 + g * 16);
+        for (int u = 0; u < 4; ++u) {
+          const bf16x8 av = *reinterpret_cast<const bf16x8*>(buf + (16 * wave + r16) * kARow + u * 64 + g * 16);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const bf16x8 av = *reinterpret_cast<const bf16x8*>(buf + (16 * j + r16) * kARow + u * 64 + g * 16);
-              acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc[j], 0, 0, 0);
-            }
+          for (int t = 0; t < MT; ++t) {
+            const bf16x8 bv = *reinterpret_cast<const bf16x8*>(buf + (16 * (waves + t) + r16) * kARow + u * 64 + g * 16);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc[t], 0, 0, 0);
           }
         }
       }
     }
   }
 
-  // lane (r16, g) holds, for row m = 16 wave + r16 of x, columns 16 j + 4 g .. + 3 of the block's 64
-  const int m = 16 * wave + r16;
-  if (!active || m >= p.m) return;
-  const bool vec = (p.n & 3) == 0 && (!GATE || (p.inter & 3) == 0);
-  if (p.splits > 1) {
-    float* out_row = p.partial + ((size_t)split * p.m + m) * p.n;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int c = 16 * j + 4 * g;
-      int col, limit;
-      if (GATE) {
-        col = tile * 32 + (c & 31) + (c >= 32 ? p.inter : 0);
-        limit = (c >= 32 ? 2 : 1) * p.inter;
-      } else {
-        col = tile * kSkinnyRows + c;
-        limit = p.n;
-      }
-      if (vec) {
-        if (col < limit) *reinterpret_cast<f32x4*>(out_row + col) = acc[j];
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (col + i < limit) out_row[col + i] = acc[j][i];
-      }
-    }
-    return;
-  }
+  // lane (r16, g) holds, for row m = 16 t + r16 of x, this wave's rows 4 g .. 4 g + 3 of w
   if (GATE) {
-    bf16_t* out_row = reinterpret_cast<bf16_t*>(p.y) + (size_t)m * p.inter;
+    const int col = col0 + 2 * g;                  // gate columns col, col + 1 in [0], [1]; their up values in [2], [3]
+    const bool pair = (p.inter & 1) == 0;          // col is even: both columns exist together, stores are aligned
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int col = tile * 32 + 16 * j + 4 * g;
-      bf16_t r[4];
+    for (int t = 0; t < MT; ++t) {
+      const int m = 16 * t + r16;
+      if (m >= p.m || col >= p.inter) continue;
+      if (p.splits > 1) {
+        float* out_row = p.partial + ((size_t)split * p.m + m) * p.n;
+        if (pair) {
+          *reinterpret_cast<float2*>(out_row + col) = float2{acc[t][0], acc[t][1]};
+          *reinterpret_cast<float2*>(out_row + p.inter + col) = float2{acc[t][2], acc[t][3]};
+        } else {
+          out_row[col] = acc[t][0];
+          out_row[p.inter + col] = acc[t][2];
+          if (col + 1 < p.inter) {
+            out_row[col + 1] = acc[t][1];
+            out_row[p.inter + col + 1] = acc[t][3];
+          }
+        }
+        continue;
+      }
+      bf16_t r[2];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float gv = acc[j][i], uv = acc[j + 2][i];
+      for (int i = 0; i < 2; ++i) {
+        float gv = acc[t][i], uv = acc[t][2 + i];
         if (p.bias && col + i < p.inter) {
           gv += p.bias[col + i];
           uv += p.bias[p.inter + col + i];
         }
         r[i] = from_f32<bf16_t>(gv / (1.f + expf(-gv)) * uv);
       }
-      if (vec) {
-        if (col < p.inter) *reinterpret_cast<uint2*>(out_row + col) = *reinterpret_cast<const uint2*>(r);
+      bf16_t* out_row = reinterpret_cast<bf16_t*>(p.y) + (size_t)m * p.inter;
+      if (pair) {
+        *reinterpret_cast<uint32_t*>(out_row + col) = *reinterpret_cast<const uint32_t*>(r);
       } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (col + i < p.inter) out_row[col + i] = r[i];
+        out_row[col] = r[0];
+        if (col + 1 < p.inter) out_row[col + 1] = r[1];
       }
     }
     return;
   }
+  const int col = col0 + 4 * g;
+  const bool vec = (p.n & 3) == 0;   // col is a multiple of 4: the four columns exist together, stores are aligned
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int col = tile * kSkinnyRows + 16 * j + 4 * g;
-    f32x4 v = acc[j];
+  for (int t = 0; t < MT; ++t) {
+    const int m = 16 * t + r16;
+    if (m >= p.m || col >= p.n) continue;
+    if (p.splits > 1) {
+      float* out_row = p.partial + ((size_t)split * p.m + m) * p.n;
+      if (vec) {
+        *reinterpret_cast<f32x4*>(out_row + col) = acc[t];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (col + i < p.n) out_row[col + i] = acc[t][i];
+      }
+      continue;
+    }
+    f32x4 v = acc[t];
     if (p.bias) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
@@ -370,7 +378,7 @@ __global__ void __launch_bounds__(256, 2) gemm_mid_kernel(SkinnyParams p) {
     if (p.out_f32) {
       float* out_row = reinterpret_cast<float*>(p.y) + (size_t)m * p.n;
       if (vec) {
-        if (col < p.n) *reinterpret_cast<f32x4*>(out_row + col) = v;
+        *reinterpret_cast<f32x4*>(out_row + col) = v;
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -382,7 +390,7 @@ __global__ void __launch_bounds__(256, 2) gemm_mid_kernel(SkinnyParams p) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) r[i] = from_f32<bf16_t>(v[i]);
       if (vec) {
-        if (col < p.n) *reinterpret_cast<uint2*>(out_row + col) = *reinterpret_cast<const uint2*>(r);
+        *reinterpret_cast<uint2*>(out_row + col) = *reinterpret_cast<const uint2*>(r);
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -423,21 +431,49 @@ static SkinnyPlan skinny_plan(int m, int tiles, int k) {
   return plan;
 }
 
-// More than 16 rows: K is cut only as far as it takes to have about 256 blocks, in slices that are a
-// multiple of the 1024 k a wave holds of x.
-static SkinnyPlan mid_plan(int tiles, int k) {
-  SkinnyPlan plan{};
+// More than 16 rows.  `groups` is the number of 16-row groups of w (8 columns each for SiLU-gate).
+// Blocks of 5 to 8 waves run one a CU, blocks of 4 waves two.  Very wide products (three rounds of
+// blocks or more whatever the choice) take four waves and K whole: with two blocks a CU one block's
+// start and end overlap another's work.  For the others the number of waves and of K slices (multiples
+// of 1024) is the one with the least work on the busiest CU: rounds of 256 blocks x rows x k a block,
+// a little more for fewer waves (x is read once per block), for every round (a block's start and end)
+// and for every slice (its partial sums are written and read again).  The choice does not depend on the number of rows of x.
+struct MidPlan {
+  int waves, tiles, splits, kslice;
+};
+
+static MidPlan mid_plan(int groups, int k) {
+  MidPlan plan{};
   const int units = (k + kMidSlice - 1) / kMidSlice;
-  int s = tiles >= 192 ? 1 : (320 + tiles - 1) / tiles;
-  s = max(1, min(s, units));
-  const int per = (units + s - 1) / s;
-  plan.kslice = per * kMidSlice;
-  plan.splits = (units + per - 1) / per;
-  plan.xk = 0;
+  if ((groups + 7) / 8 > 2 * 256) {
+    plan.waves = 4;
+    plan.tiles = (groups + 3) / 4;
+    plan.splits = 1;
+    plan.kslice = units * kMidSlice;
+    return plan;
+  }
+  double best = 1e30;
+  for (int s = 1; s <= min(units, 32); ++s) {
+    const int per = (units + s - 1) / s;
+    const int splits = (units + per - 1) / per;
+    if (splits != s) continue;
+    for (int w = 8; w >= 4; --w) {
+      const long tiles = (groups + w - 1) / w;
+      const long rounds = (tiles * splits + 255) / 256;
+      const double cost = (double)rounds * w * per * (1. + 1. / w) + 0.5 * rounds + 0.15 * splits * groups / 256.;
+      if (cost < best - 1e-9) {
+        best = cost;
+        plan.waves = w;
+        plan.tiles = (int)tiles;
+        plan.splits = splits;
+        plan.kslice = per * kMidSlice;
+      }
+    }
+  }
   return plan;
 }
 
-static SkinnyPlan plan_for(int m, int tiles, int k) { return m > 16 ? mid_plan(tiles, k) : skinny_plan(m, tiles, k); }
+static int mid_groups(int n, int gate) { return gate ? (n + 7) / 8 : (n + 15) / 16; }
 
 // 1 if the skinny kernel takes this product.
 ATOM_EXPORT int atom_gemm_skinny_supports(int m, int n, int k) {
@@ -446,7 +482,8 @@ ATOM_EXPORT int atom_gemm_skinny_supports(int m, int n, int k) {
 
 // Into how many slices atom_gemm_skinny cuts K for this product (1: it writes y itself).
 ATOM_EXPORT int atom_gemm_skinny_splits(int m, int n, int k, int gate) {
-  return plan_for(max(m, 1), skinny_tiles(n, gate), k).splits;
+  if (m > 16) return mid_plan(mid_groups(n, gate), k).splits;
+  return skinny_plan(max(m, 1), skinny_tiles(n, gate), k).splits;
 }
 
 // gate == 0: x w^T, n columns.  gate == 1: w is [2 n, k] (n gate rows, then n up rows).
@@ -465,34 +502,50 @@ ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias
   p.m = m; p.k = k; p.out_f32 = out_f32;
   p.n = gate ? 2 * n : n;
   p.inter = gate ? n : 0;
+  const int mt = (m + 15) / 16;
+  if (m > 16) {
+    if ((uintptr_t)y & 15) return ATOM_BAD_SHAPE;
+    const MidPlan plan = mid_plan(mid_groups(n, gate), k);
+    p.tiles = plan.tiles; p.splits = plan.splits; p.kslice = plan.kslice;
+    if (p.splits > 1 ? partial == nullptr : y == nullptr) return ATOM_BAD_SHAPE;
+    const long blocks = (long)p.tiles * p.splits;
+    if (blocks > 0x7fffffffL) return ATOM_TOO_LARGE;
+    const size_t lds = (size_t)2 * (16 * plan.waves + 16 * mt) * kARow;
+    // two chunks of LDS are more than a launch gets by default: allow it once per kernel
+#define GO_MID(MTV, G)                                                                                     \
+  do {                                                                                                     \
+    static bool allowed = false;                                                                           \
+    if (!allowed) {                                                                                        \
+      if (hipFuncSetAttribute((const void*)gemm_mid_kernel<MTV, G>,                                        \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 2 * (16 * 8 + 64) * kARow) !=    \
+          hipSuccess)                                                                                      \
+        return ATOM_LAUNCH_FAILED;                                                                         \
+      allowed = true;                                                                                      \
+    }                                                                                                      \
+    hipLaunchKernelGGL((gemm_mid_kernel<MTV, G>), dim3(blocks), dim3(64 * plan.waves), lds, stream, p);    \
+  } while (0)
+#define GO(MTV)                      \
+  do {                               \
+    if (gate) GO_MID(MTV, true);     \
+    else GO_MID(MTV, false);         \
+  } while (0)
+    switch (mt) {
+      case 2: GO(2); break;
+      case 3: GO(3); break;
+      default: GO(4); break;
+    }
+#undef GO
+#undef GO_MID
+    return launch_status();
+  }
   p.tiles = skinny_tiles(n, gate);
-  const SkinnyPlan plan = plan_for(m, p.tiles, k);
+  const SkinnyPlan plan = skinny_plan(m, p.tiles, k);
   p.splits = plan.splits; p.kslice = plan.kslice; p.xk = plan.xk;
   if (p.splits > 1 ? partial == nullptr : y == nullptr) return ATOM_BAD_SHAPE;
   const long blocks = (long)p.tiles * p.splits;
   if (blocks > 0x7fffffffL) return ATOM_TOO_LARGE;
-  if (m > 16) {
-    if ((uintptr_t)y & 15) return ATOM_BAD_SHAPE;
-    // two chunks of LDS are more than a launch gets by default: allow it once per kernel
-#define GO_MID(G)                                                                                          \
-  do {                                                                                                     \
-    static bool allowed = false;                                                                           \
-    if (!allowed) {                                                                                        \
-      if (hipFuncSetAttribute((const void*)gemm_mid_kernel<G>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                              2 * kMidBuf) != hipSuccess)                                                  \
-        return ATOM_LAUNCH_FAILED;                                                                         \
-      allowed = true;                                                                                      \
-    }                                                                                                      \
-    hipLaunchKernelGGL(gemm_mid_kernel<G>, dim3(blocks), dim3(256), 2 * kMidBuf, stream, p);               \
-  } while (0)
-    if (gate) GO_MID(true);
-    else GO_MID(false);
-#undef GO_MID
-    return launch_status();
-  }
   const size_t lds = (size_t)4 * kAWave + max((size_t)m * (p.xk * 2 + 16), (size_t)m * (kSkinnyRows + 1) * 4);
-  const int mt = (m + 15) / 16;
-  // 64 rows of x need a little more LDS than a launch gets by default: allow it once per kernel
+  // a long slice of x needs more LDS than a launch gets by default: allow it once per kernel
 #define GO_ONE(MTV, G)                                                                                   \
   do {                                                                                                   \
     static bool allowed = false;                                                                         \
@@ -509,12 +562,7 @@ ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias
     if (gate) GO_ONE(MTV, true);     \
     else GO_ONE(MTV, false);         \
   } while (0)
-  switch (mt) {
-    case 1: GO(1); break;
-    case 2: GO(2); break;
-    case 3: GO(3); break;
-    default: GO(4); break;
-  }
+  GO(1);
 #undef GO
 #undef GO_ONE
   return launch_status();
