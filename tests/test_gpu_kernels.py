@@ -502,7 +502,7 @@ def test_kernels_refuse_what_they_cannot_take():
 
 @pytest.fixture
 def all_rows():
-    """The skinny kernel for every row count it takes (the engine hands it at most 16 rows)."""
+    """The skinny kernels for every row count they take."""
     ops = gpu_ops()
     before = ops.skinny_max_rows
     ops.skinny_max_rows = 64

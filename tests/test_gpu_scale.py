@@ -104,8 +104,8 @@ def test_cuts_agree_at_serving_sizes():
 
 
 def test_many_live_requests_decode_like_each_alone():
-    """48 requests of different lengths decode together (the library's products, attention parts merged
-    inside a block); each row equals the request decoded alone (the skinny kernel, the merge kernel)."""
+    """48 requests of different lengths decode together (the product kernel for 17 to 64 rows, attention parts
+    merged inside a block); each row equals the request decoded alone (the kernel for up to 16 rows, the merge kernel)."""
     core = _core(torch.bfloat16, graph_sizes=[1, 64], num_pages=4096)
     lens = [17 + 53 * k for k in range(48)]
     prompts = {f"r{k}": _ids(n, 100 + k) for k, n in enumerate(lens)}
