@@ -223,6 +223,7 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
 // SiLU-gate: a wave's 16 rows are 8 gate and 8 up rows of the same 8 columns, ordered so that a lane's
 // four results are two gate values and the two up values of the same columns.
 constexpr int kMidSlice = 1024;   // K is cut in multiples of this
+constexpr int kMidAhead = 4;      // chunks in flight a wave (3 and 5 measure the same)
 
 template <int MT, bool GATE>
 __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
@@ -265,27 +266,34 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
   f32x4 acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  bf16x8 a[16], xa[16];
-  auto load_chunk = [&](int slot, int ci) {
+  bf16x8 a[4 * kMidAhead], xa[4 * kMidAhead];
+  auto load_w = [&](int slot, int ci) {
     const int kk = k_begin + 128 * ci;
     const bool in = kk + 8 * r16 < k_end;
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg)
       a[4 * slot + rg] = in ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[rg] + kk)) : zero;
+  };
+  auto load_x = [&](int slot, int ci) {
+    const int kk = k_begin + 128 * ci;
+    const bool in = kk + 8 * r16 < k_end;
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg)
       if (xmine[rg]) xa[4 * slot + rg] = in ? *reinterpret_cast<const bf16x8*>(xrow[rg] + kk) : zero;
   };
 #pragma unroll
-  for (int slot = 0; slot < 4; ++slot)
-    if (slot < total) load_chunk(slot, slot);
+  for (int slot = 0; slot < kMidAhead; ++slot)
+    if (slot < total) {
+      load_w(slot, slot);
+      load_x(slot, slot);
+    }
 
-  for (int base = 0; base < total; base += 4) {
+  for (int base = 0; base < total; base += kMidAhead) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
+    for (int c = 0; c < kMidAhead; ++c) {
       const int ci = base + c;
       if (ci < total) {   // the same in every wave of the block
-        char* buf = lds + (c & 1) * chunk_bytes;
+        char* buf = lds + (ci & 1) * chunk_bytes;
         // the two buffers take turns: a wave that writes chunk ci has passed the barrier of chunk ci - 1,
         // which every wave reaches only after it has read chunk ci - 2
 #pragma unroll
@@ -294,7 +302,10 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg)
           if (xmine[rg]) *reinterpret_cast<bf16x8*>(buf + xat[rg]) = xa[4 * c + rg];
-        if (ci + 4 < total) load_chunk(c, ci + 4);
+        if (ci + kMidAhead < total) {
+          load_w(c, ci + kMidAhead);
+          load_x(c, ci + kMidAhead);
+        }
         __syncthreads();
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
