@@ -513,7 +513,8 @@ def all_rows():
 @pytest.mark.parametrize("m,n,k", [(1, 311, 136), (8, 4096, 4096), (16, 517, 200), (17, 1000, 520), (33, 96, 2056),
                                    (64, 640, 1032), (5, 64, 8), (3, 6144, 4096), (7, 130, 12288),
                                    (3, 16400, 520), (40, 16390, 1032), (8, 20000, 4096), (64, 16384, 2056),
-                                   (20, 32768, 264), (50, 28672, 136), (30, 24570, 520)])
+                                   (20, 32768, 264), (50, 28672, 136), (30, 24570, 520),
+                                   (18, 3, 8), (64, 7, 40), (47, 130, 12288), (17, 4098, 4096)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_skinny_gemm(m, n, k, out_dtype, all_rows):
     ops = all_rows
@@ -556,7 +557,7 @@ def test_skinny_gemm_is_what_runs():
 
 @pytest.mark.parametrize("m,inter,k", [(1, 200, 136), (8, 12288, 4096), (20, 333, 264), (64, 160, 96),
                                        (33, 8200, 1032), (64, 8192, 4096), (24, 14336, 136), (48, 12287, 264),
-                                       (17, 16384, 72)])
+                                       (17, 16384, 72), (18, 3, 8), (40, 6, 16), (64, 1001, 2056)])
 def test_skinny_gemm_silu_gate(m, inter, k, all_rows):
     ops = all_rows
     x = rnd((m, k), torch.bfloat16, 50, 1.0)
