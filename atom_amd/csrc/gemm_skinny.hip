@@ -1,4 +1,4 @@
-// y[M, N] = x[M, K] * w[N, K]^T (+ bias) for few rows (M <= 64), bfloat16 operands,
+// y[M, N] = x[M, K] * w[N, K]^T (+ bias) for few rows (M <= 64; narrow products M <= 128), bfloat16 operands,
 // float32 accumulation on the matrix cores.  This is the decode-step product: the
 // weight matrix is streamed from memory once and the work is bound by that stream.
 //
@@ -24,7 +24,8 @@
 // SiLU-gate: w holds `inter` gate rows then `inter` up rows, a block owns 32 columns of
 // each, and writes silu(gate) * up [M, inter].
 //
-// Needs K % 8 == 0 (16-byte loads).  Any N, any M <= 64.
+// Needs K % 8 == 0 (16-byte loads).  Any N, any M <= 64; atom_gemm_skinny_supports says which products
+// with up to 128 rows it takes.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -37,6 +38,7 @@ struct SkinnyParams {
   void* y;             // splits == 1: [m, n] bfloat16 or float32 (gate: [m, inter] bfloat16)
   float* partial;      // splits > 1: [splits, m, n]
   int m, n, k, inter, out_f32, splits, tiles, kslice, xk;
+  int halves, rows_half;   // 65 to 128 rows: two blocks share a tile of w, each with rows_half rows of x
 };
 
 struct SkinnyPlan {
@@ -222,6 +224,10 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
 //
 // SiLU-gate: a wave's 16 rows are 8 gate and 8 up rows of the same 8 columns, ordered so that a lane's
 // four results are two gate values and the two up values of the same columns.
+//
+// 65 to 128 rows of x, for products whose blocks of four waves all fit on the chip twice over: every
+// block comes twice, side by side in the grid, each with half of the rows of x.  The pair reads its
+// rows of w at about the same time, so memory delivers them once.
 constexpr int kMidSlice = 1024;   // K is cut in multiples of this
 constexpr int kMidAhead = 4;      // chunks in flight a wave (3 and 5 measure the same)
 
@@ -235,8 +241,12 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
   const int r16 = lane & 15;
   const int g = lane >> 4;
   const int k = p.k;
-  const int tile = blockIdx.x / p.splits;
-  const int split = blockIdx.x - tile * p.splits;
+  // with more than 64 rows of x neighbouring blocks take the same rows of w and a half of x each
+  const int unit = blockIdx.x / p.halves;
+  const int m_base = (blockIdx.x - unit * p.halves) * p.rows_half;
+  const int m_rows = min(p.rows_half, p.m - m_base);
+  const int tile = unit / p.splits;
+  const int split = unit - tile * p.splits;
   const int k_begin = split * p.kslice;
   const int k_end = min(k, k_begin + p.kslice);
   const int total = (k_end - k_begin + 127) / 128;   // chunks
@@ -259,7 +269,7 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
     const int four = wave + waves * rg;   // which four rows of x
     xmine[rg] = four < 4 * MT;
     xat[rg] = (16 * waves + 4 * four + g) * kARow + r16 * 16;
-    xrow[rg] = p.x + (size_t)min(4 * four + g, p.m - 1) * k + 8 * r16;
+    xrow[rg] = p.x + (size_t)(m_base + min(4 * four + g, m_rows - 1)) * k + 8 * r16;
   }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
@@ -320,14 +330,14 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
     }
   }
 
-  // lane (r16, g) holds, for row m = 16 t + r16 of x, this wave's rows 4 g .. 4 g + 3 of w
+  // lane (r16, g) holds, for row 16 t + r16 of the block's rows of x, this wave's rows 4 g .. 4 g + 3 of w
   if (GATE) {
     const int col = col0 + 2 * g;                  // gate columns col, col + 1 in [0], [1]; their up values in [2], [3]
     const bool pair = (p.inter & 1) == 0;          // col is even: both columns exist together, stores are aligned
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      const int m = 16 * t + r16;
-      if (m >= p.m || col >= p.inter) continue;
+      if (16 * t + r16 >= m_rows || col >= p.inter) continue;
+      const int m = m_base + 16 * t + r16;
       if (p.splits > 1) {
         float* out_row = p.partial + ((size_t)split * p.m + m) * p.n;
         if (pair) {
@@ -367,8 +377,8 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
   const bool vec = (p.n & 3) == 0;   // col is a multiple of 4: the four columns exist together, stores are aligned
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
-    const int m = 16 * t + r16;
-    if (m >= p.m || col >= p.n) continue;
+    if (16 * t + r16 >= m_rows || col >= p.n) continue;
+    const int m = m_base + 16 * t + r16;
     if (p.splits > 1) {
       float* out_row = p.partial + ((size_t)split * p.m + m) * p.n;
       if (vec) {
@@ -488,7 +498,11 @@ static int mid_groups(int n, int gate) { return gate ? (n + 7) / 8 : (n + 15) / 
 
 // 1 if the skinny kernel takes this product.
 ATOM_EXPORT int atom_gemm_skinny_supports(int m, int n, int k) {
-  return m >= 1 && m <= 64 && n >= 1 && k >= 8 && k % 8 == 0;
+  if (m < 1 || n < 1 || k < 8 || k % 8) return 0;
+  if (m <= 64) return 1;
+  if (m > 128) return 0;
+  const MidPlan plan = mid_plan(mid_groups(n, 0), k);   // the same groups with SiLU-gate: n is then twice the columns
+  return plan.waves == 4 && plan.tiles * plan.splits <= 256;
 }
 
 // Into how many slices atom_gemm_skinny cuts K for this product (1: it writes y itself).
@@ -504,7 +518,7 @@ ATOM_EXPORT int atom_gemm_skinny_splits(int m, int n, int k, int gate) {
 ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias, void* y, float* partial,
                                  int m, int n, int k, int out_f32, int gate, hipStream_t stream) {
   if (m < 0 || n <= 0 || k <= 0) return ATOM_BAD_SHAPE;
-  if (m > 64 || k % 8) return ATOM_UNSUPPORTED;
+  if (k % 8 || !atom_gemm_skinny_supports(max(m, 1), gate ? 2 * n : n, k)) return ATOM_UNSUPPORTED;
   if (gate && out_f32) return ATOM_UNSUPPORTED;
   if (m == 0) return ATOM_OK;
   if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)partial) & 15) return ATOM_BAD_SHAPE;
@@ -513,13 +527,15 @@ ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias
   p.m = m; p.k = k; p.out_f32 = out_f32;
   p.n = gate ? 2 * n : n;
   p.inter = gate ? n : 0;
-  const int mt = (m + 15) / 16;
+  p.halves = m > 64 ? 2 : 1;
+  p.rows_half = ((m + p.halves - 1) / p.halves + 15) / 16 * 16;
+  const int mt = p.rows_half / 16;
   if (m > 16) {
     if ((uintptr_t)y & 15) return ATOM_BAD_SHAPE;
     const MidPlan plan = mid_plan(mid_groups(n, gate), k);
     p.tiles = plan.tiles; p.splits = plan.splits; p.kslice = plan.kslice;
     if (p.splits > 1 ? partial == nullptr : y == nullptr) return ATOM_BAD_SHAPE;
-    const long blocks = (long)p.tiles * p.splits;
+    const long blocks = (long)p.tiles * p.splits * p.halves;
     if (blocks > 0x7fffffffL) return ATOM_TOO_LARGE;
     const size_t lds = (size_t)2 * (16 * plan.waves + 16 * mt) * kARow;
     // two chunks of LDS are more than a launch gets by default: allow it once per kernel

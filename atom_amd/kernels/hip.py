@@ -121,7 +121,7 @@ class HipKernels:
         # bfloat16 products of few rows run this library's own weight-streaming kernel.  It takes up to 64
         # rows; beyond 16 (one matrix-core tile of rows) the BLAS library's kernels are faster on gfx950.
         self.use_skinny_gemm = True
-        self.skinny_max_rows = 64
+        self.skinny_max_rows = 128
         self.use_mfma_attention = True
         self.use_tiled_prefill = True
         self._ws: dict[str, torch.Tensor] = {}
@@ -392,8 +392,8 @@ class HipKernels:
                     and weight.dtype == torch.bfloat16 and self.lib.atom_gemm_skinny_supports(m, weight.shape[0], k))
 
     def linear(self, x, weight, bias=None, out_dtype=None, defer: bool = False):
-        """``x @ weight.T (+ bias)``.  bfloat16 operands with at most 64 rows run this library's own
-        weight-streaming kernel; with more rows they go to the BLAS library, as the reference's engine
+        """``x @ weight.T (+ bias)``.  bfloat16 operands with at most 64 rows (narrow products: 128) run this
+        library's own weight-streaming kernels; with more rows they go to the BLAS library, as the reference's engine
         does for its matrix products; anything with a float32 operand runs this library's float32
         kernel (plain FMA, no reduced-precision mode).  With ``defer`` the result may come back as a
         ``DeferredSum`` for a kernel that adds the slices while it reads them."""

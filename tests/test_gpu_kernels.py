@@ -505,7 +505,7 @@ def all_rows():
     """The skinny kernels for every row count they take."""
     ops = gpu_ops()
     before = ops.skinny_max_rows
-    ops.skinny_max_rows = 64
+    ops.skinny_max_rows = 128
     yield ops
     ops.skinny_max_rows = before
 
@@ -514,7 +514,8 @@ def all_rows():
                                    (64, 640, 1032), (5, 64, 8), (3, 6144, 4096), (7, 130, 12288),
                                    (3, 16400, 520), (40, 16390, 1032), (8, 20000, 4096), (64, 16384, 2056),
                                    (20, 32768, 264), (50, 28672, 136), (30, 24570, 520),
-                                   (18, 3, 8), (64, 7, 40), (47, 130, 12288), (17, 4098, 4096)])
+                                   (18, 3, 8), (64, 7, 40), (47, 130, 12288), (17, 4098, 4096),
+                                   (65, 96, 2056), (100, 640, 1032), (128, 4096, 4096), (97, 130, 12288), (81, 5, 8)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_skinny_gemm(m, n, k, out_dtype, all_rows):
     ops = all_rows
@@ -543,7 +544,7 @@ def test_skinny_gemm(m, n, k, out_dtype, all_rows):
 
 
 def test_skinny_gemm_is_what_runs():
-    """At most 64 bfloat16 rows take the engine's own kernel, not the library."""
+    """Few bfloat16 rows take the engine's own kernel, not the library."""
     ops = gpu_ops()
     x = rnd((8, 512), torch.bfloat16, 1).to(DEV)
     w = rnd((256, 512), torch.bfloat16, 2, 0.05).to(DEV)
@@ -557,7 +558,8 @@ def test_skinny_gemm_is_what_runs():
 
 @pytest.mark.parametrize("m,inter,k", [(1, 200, 136), (8, 12288, 4096), (20, 333, 264), (64, 160, 96),
                                        (33, 8200, 1032), (64, 8192, 4096), (24, 14336, 136), (48, 12287, 264),
-                                       (17, 16384, 72), (18, 3, 8), (40, 6, 16), (64, 1001, 2056)])
+                                       (17, 16384, 72), (18, 3, 8), (40, 6, 16), (64, 1001, 2056),
+                                       (128, 160, 96), (70, 333, 264)])
 def test_skinny_gemm_silu_gate(m, inter, k, all_rows):
     ops = all_rows
     x = rnd((m, k), torch.bfloat16, 50, 1.0)
