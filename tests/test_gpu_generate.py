@@ -162,6 +162,45 @@ def test_steps_launched_ahead_change_no_token(dtype):
     assert llm.is_finished() and not llm.core.manager.live_requests()
 
 
+def test_steps_launched_ahead_under_random_load_on_the_gpu():
+    """Requests of random lengths and token counts arrive while others run, some end on a token, the pool is
+    small enough to preempt, prompts share beginnings (prefix cache).  In 32-bit a row's logits do not depend on
+    the batch to the bit, so with and without steps launched ahead every request gets the same tokens."""
+    import random
+
+    rng = random.Random(3)
+    shared = random_ids("A", 24, 700)
+    arrivals = []
+    for k in range(12):
+        body = random_ids("A", rng.randrange(1, 30), 800 + k)
+        prompt = (shared[:rng.choice([0, 16, 24])] + body)[:60]
+        sp = SamplingParams(temperature=rng.choice([0.0, 0.0, 0.8]), max_tokens=rng.randrange(1, 40), seed=k,
+                            ignore_eos=rng.random() < 0.5)
+        arrivals.append((rng.randrange(0, 25), prompt, sp))
+    arrivals.sort(key=lambda a: a[0])
+
+    def run(deferred):
+        llm = engine("A", "fp32", num_kvcache_blocks=6, max_num_seqs=3, eos_token_id=7, max_model_len=128,
+                     stop_token_ids=list(range(0, 256, 16)), deferred_output=deferred)
+        seqs, outputs, pending, step = {}, {}, list(arrivals), 0
+        while pending or not llm.is_finished():
+            while pending and pending[0][0] <= step:
+                _, prompt, sp = pending.pop(0)
+                seqs[llm.add_request(prompt, sp)[0].id] = len(seqs)
+            for seq in llm.step():
+                outputs[seqs[seq.id]] = (seq.completion_token_ids, seq.leave_reason)
+            llm.core.manager.check()
+            step += 1
+            assert step < 2000
+        assert not llm.core.manager.live_requests()
+        return outputs, llm
+
+    waited, _ = run(False)
+    ahead, llm = run(True)
+    assert len(waited) == len(arrivals) and ahead == waited
+    assert llm.scheduler.total_preemptions > 0 and llm.core.graphs.replays > 10
+
+
 def test_mark_trace_names_the_operations_in_a_profile():
     """With mark_trace the steps' spans hold one span per operation, and the tokens do not change."""
     from atom_amd.kernels.hip import HipKernels
