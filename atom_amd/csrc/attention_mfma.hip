@@ -767,22 +767,37 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
   // ---- moving a tile: piece q of K is (key q / (D/8), 8 elements at (q % (D/8)) * 8);
   //      piece q of V^T is (d = q / (TK/8), the 8 keys at (q % (TK/8)) * 8)
   bf16x8 kreg[PT], vreg[PT];
-  const size_t page_elems = (size_t)p.hkv * ps * D;        // elements of a page, all heads
+  const uint32_t page_elems = (uint32_t)p.hkv * ps * D;    // elements of a page, all heads
   const int k_head = kvh * ps * D, v_head = kvh * D * ps;  // this KV head's part of a key page and of a value page
+  // The pages of a tile are looked up a tile before its loads go out (`pages_of`), so that no load waits for a
+  // table entry; a thread's pieces of V^T all lie in one page (256 is a multiple of the pieces per row).
+  static_assert(256 % (TK / 8) == 0, "a thread's V^T pieces must share their keys");
+  int kpage[PT], vpage = 0;
+  auto pages_of_as = [&](int k0, auto kind) {
+    const PageMath<decltype(kind)::value> pages{ps, p.page_shift};
+#pragma unroll
+    for (int j = 0; j < PT; ++j) {
+      const int key = min(k0 + (tid + 256 * j) / (D / 8), ke - 1);
+      kpage[j] = table[pages.index(key)];
+    }
+    const int vkey = min(k0 + (tid % (TK / 8)) * 8, (ke - 1) & ~7);
+    vpage = table[pages.index(vkey)];
+  };
+  auto pages_of = [&](int k0) {
+    if (p.page_shift >= 0) pages_of_as(k0, Pow2Pages{});
+    else pages_of_as(k0, AnyPages{});
+  };
   auto load_tile_as = [&](int k0, auto kind) {
     const PageMath<decltype(kind)::value> pages{ps, p.page_shift};
+    const int vkey = min(k0 + (tid % (TK / 8)) * 8, (ke - 1) & ~7);
+    const bf16_t* vbase = p.v_cache + (uint64_t)(uint32_t)vpage * page_elems + (v_head + pages.within(vkey));
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
       const int q = tid + 256 * j;
       const int key = min(k0 + q / (D / 8), ke - 1);
-      const int page = table[pages.index(key)];
-      kreg[j] = *reinterpret_cast<const bf16x8*>(p.k_cache + page * page_elems +
+      kreg[j] = *reinterpret_cast<const bf16x8*>(p.k_cache + (uint64_t)(uint32_t)kpage[j] * page_elems +
                                                  (k_head + pages.within(key) * D + (q % (D / 8)) * 8));
-      const int d = q / (TK / 8);
-      const int vkey = min(k0 + (q % (TK / 8)) * 8, (ke - 1) & ~7);
-      const int vpage = table[pages.index(vkey)];
-      vreg[j] = *reinterpret_cast<const bf16x8*>(p.v_cache + vpage * page_elems +
-                                                 (v_head + d * ps + pages.within(vkey)));
+      vreg[j] = *reinterpret_cast<const bf16x8*>(vbase + (q / (TK / 8)) * ps);
     }
   };
   auto load_tile = [&](int k0) {
@@ -808,12 +823,19 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
     }
   };
 
-  if (kb < ke) load_tile(kb);
+  if (kb < ke) {
+    pages_of(kb);
+    load_tile(kb);
+    if (kb + TK < ke) pages_of(kb + TK);
+  }
   for (int k0 = kb; k0 < ke; k0 += TK) {
     __syncthreads();   // the previous tile has been read by every wave
     store_tile();
     __syncthreads();
-    if (k0 + TK < ke) load_tile(k0 + TK);
+    if (k0 + TK < ke) {
+      load_tile(k0 + TK);
+      if (k0 + 2 * TK < ke) pages_of(k0 + 2 * TK);
+    }
     if (nrows == 0 || k0 >= my_ke) continue;   // the whole wave: nothing of this tile is visible to it
 
     // ---- S^T for the blocks of 16 keys
@@ -822,10 +844,11 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int b = 0; b < KB; ++b) s[rt][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // (the head-size chunks outermost: successive products go to different accumulators)
 #pragma unroll
-    for (int b = 0; b < KB; ++b)
+    for (int j = 0; j < KCH; ++j)
 #pragma unroll
-      for (int j = 0; j < KCH; ++j) {
+      for (int b = 0; b < KB; ++b) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks + (16 * b + r16) * KSTR + 32 * j + 8 * g);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
