@@ -51,6 +51,7 @@ constexpr int kSkinnyLds = 64 * 1024;
 constexpr int kARow = 256 + 16;    // LDS bytes of one row of a quarter shot (128 k), padded by 4 banks
 constexpr int kAWave = 16 * kARow; // LDS bytes of a wave's layout-change area
 
+// MT: 16-row tiles of x; launched with one (more rows go to gemm_mid_kernel).
 template <int MT, bool GATE>
 __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
   constexpr int THREADS = 256;
