@@ -61,6 +61,21 @@ def test_long_decoding_past_the_window_and_many_pages():
     check_greedy("C", "fp32", [prompt], [out])
 
 
+@pytest.mark.parametrize("live", [40, 100])
+def test_many_requests_decode_together(live):
+    """40 and 100 live requests in bfloat16: decode steps of 17 to 64 and of 65 to 128 rows (the product
+    kernels for those row counts, the graph buckets above 32); every token is the plain argmax within rounding."""
+    prompts = [random_ids("B", 3 + (7 * k) % 40, 300 + k) for k in range(live)]
+    llm = engine("B", "bf16", max_num_seqs=128, num_kvcache_blocks=1024,
+                 cudagraph_capture_sizes=[1, 2, 4, 8, 16, 32, 48, 64, 128])
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True))
+    assert llm.core.graphs.replays >= 3
+    picks = list(range(0, live, 7))
+    check_greedy("B", "bf16", [prompts[k] for k in picks], [outs[k] for k in picks])
+    llm.core.manager.check()
+    assert not llm.core.manager.live_requests()
+
+
 def test_first_tokens_of_a_sequence():
     """Prompts of one and two tokens: the first position has a single key, itself."""
     for which in ("A", "B"):
