@@ -232,7 +232,9 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
 constexpr int kMidSlice = 1024;   // K is cut in multiples of this
 constexpr int kMidAhead = 4;      // chunks in flight a wave (3 and 5 measure the same)
 
-template <int MT, bool GATE>
+// EXACT: the block's range of K is whole chunks, so no load needs a guard.  TURN: K is not cut, and every
+// tile starts its walk through K at another eighth.
+template <int MT, bool GATE, bool EXACT, bool TURN>
 __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
   extern __shared__ __attribute__((aligned(16))) char lds[];   // two chunks of 16 W + 16 MT rows
   const int tid = threadIdx.x;
@@ -252,6 +254,15 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
   const int k_end = min(k, k_begin + p.kslice);
   const int total = (k_end - k_begin + 127) / 128;   // chunks
   const int chunk_bytes = (16 * waves + 16 * MT) * kARow;
+  // Blocks that start together would all read the same stretch of their rows, a row's length apart in memory,
+  // and so the same few memory channels at any moment: where K is not cut (slices start apart anyway, and
+  // measure worse with this) every tile starts its walk through K at another eighth.
+  const int first = (TURN && total >= 8) ? (tile & 7) * (total >> 3) : 0;
+  auto k_of = [&](int ci) {
+    if (!TURN) return k_begin + 128 * ci;
+    const int c = ci + first;
+    return k_begin + 128 * (c < total ? c : c - total);
+  };
 
   // first column of this wave; row j (0..15) of the wave in w
   const int col0 = GATE ? (tile * waves + wave) * 8 : (tile * waves + wave) * 16;
@@ -279,15 +290,15 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
   for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   bf16x8 a[4 * kMidAhead], xa[4 * kMidAhead];
   auto load_w = [&](int slot, int ci) {
-    const int kk = k_begin + 128 * ci;
-    const bool in = kk + 8 * r16 < k_end;
+    const int kk = k_of(ci);
+    const bool in = EXACT || kk + 8 * r16 < k_end;
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg)
       a[4 * slot + rg] = in ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[rg] + kk)) : zero;
   };
   auto load_x = [&](int slot, int ci) {
-    const int kk = k_begin + 128 * ci;
-    const bool in = kk + 8 * r16 < k_end;
+    const int kk = k_of(ci);
+    const bool in = EXACT || kk + 8 * r16 < k_end;
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg)
       if (xmine[rg]) xa[4 * slot + rg] = in ? *reinterpret_cast<const bf16x8*>(xrow[rg] + kk) : zero;
@@ -540,29 +551,39 @@ ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias
     if (blocks > 0x7fffffffL) return ATOM_TOO_LARGE;
     const size_t lds = (size_t)2 * (16 * plan.waves + 16 * mt) * kARow;
     // two chunks of LDS are more than a launch gets by default: allow it once per kernel
-#define GO_MID(MTV, G)                                                                                     \
+#define GO_MID(MTV, G, E, T)                                                                                    \
   do {                                                                                                     \
     static bool allowed = false;                                                                           \
     if (!allowed) {                                                                                        \
-      if (hipFuncSetAttribute((const void*)gemm_mid_kernel<MTV, G>,                                        \
+      if (hipFuncSetAttribute((const void*)gemm_mid_kernel<MTV, G, E, T>,                                        \
                               hipFuncAttributeMaxDynamicSharedMemorySize, 2 * (16 * 8 + 64) * kARow) !=    \
           hipSuccess)                                                                                      \
         return ATOM_LAUNCH_FAILED;                                                                         \
       allowed = true;                                                                                      \
     }                                                                                                      \
-    hipLaunchKernelGGL((gemm_mid_kernel<MTV, G>), dim3(blocks), dim3(64 * plan.waves), lds, stream, p);    \
+    hipLaunchKernelGGL((gemm_mid_kernel<MTV, G, E, T>), dim3(blocks), dim3(64 * plan.waves), lds, stream, p);    \
   } while (0)
-#define GO(MTV)                      \
-  do {                               \
-    if (gate) GO_MID(MTV, true);     \
-    else GO_MID(MTV, false);         \
+#define GO_E(MTV, G, E)                  \
+  do {                                   \
+    if (turn) GO_MID(MTV, G, E, true);   \
+    else GO_MID(MTV, G, E, false);       \
   } while (0)
+#define GO(MTV)                               \
+  do {                                        \
+    if (gate && exact) GO_E(MTV, true, true); \
+    else if (gate) GO_E(MTV, true, false);    \
+    else if (exact) GO_E(MTV, false, true);   \
+    else GO_E(MTV, false, false);             \
+  } while (0)
+    const bool turn = p.splits == 1;
+    const bool exact = k % 128 == 0;   // slices are multiples of 1024
     switch (mt) {
       case 2: GO(2); break;
       case 3: GO(3); break;
       default: GO(4); break;
     }
 #undef GO
+#undef GO_E
 #undef GO_MID
     return launch_status();
   }
