@@ -2,7 +2,9 @@
 // float32 accumulation on the matrix cores.  This is the decode-step product: the
 // weight matrix is streamed from memory once and the work is bound by that stream.
 //
-// Up to 16 rows of x (gemm_skinny_kernel; 17 to 64 rows: gemm_mid_kernel, described at its place).
+// Two kernels: gemm_skinny_kernel, described here, stages the block's slice of x in LDS and takes up to 16
+// rows of x; gemm_mid_kernel, described at its place, streams x beside the weights and takes up to 64 (128).
+// takes_mid() says which one runs.
 // A block of four waves owns 64 rows of w (64 output columns) and a slice of K; each
 // wave owns 16 of the rows and walks its part of the slice in shots of 512 k.  For a shot
 // a wave issues all its 16 loads at once, non-temporal, each covering 256 contiguous
@@ -51,7 +53,7 @@ constexpr int kSkinnyLds = 64 * 1024;
 constexpr int kARow = 256 + 16;    // LDS bytes of one row of a quarter shot (128 k), padded by 4 banks
 constexpr int kAWave = 16 * kARow; // LDS bytes of a wave's layout-change area
 
-// MT: 16-row tiles of x; launched with one (more rows go to gemm_mid_kernel).
+// MT: 16-row tiles of x; launched with one.
 template <int MT, bool GATE>
 __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
   constexpr int THREADS = 256;
@@ -214,8 +216,8 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
   }
 }
 
-// ---- 17 to 64 rows of x.  With that many rows a useful slice of x no longer fits in LDS beside the
-// weights' layout-change areas, so x is streamed like the weights.  A block of W waves (4 to 8) owns
+// ---- Up to 64 rows of x (needed from 17 rows on: with that many a useful slice of x no longer fits in LDS
+// beside the weights' layout-change areas), x streamed like the weights.  A block of W waves (4 to 8) owns
 // 16 W rows of w and a range of K; a chunk is 128 k of those rows and of the rows of x.  Each wave loads
 // its own 16 rows of w and a share of the rows of x (the same whole-cache-line loads as above, four
 // chunks in flight a wave) and writes them to one of two LDS buffers; after the block's barrier it
@@ -506,6 +508,11 @@ static MidPlan mid_plan(int groups, int k) {
   return plan;
 }
 
+// Which of the two kernels takes a product.  Measured on an MI355X with the Qwen3-8B products: the streaming
+// kernel is the faster one from 9 rows on, and for SiLU-gate from the first row (it does not cut K there, so
+// the gate is applied in place and no second kernel reads partial sums); with up to 8 rows the kernel that
+// stages x is equal or a little faster for the plain products.
+static bool takes_mid(int m, int gate) { return gate || m > 8; }
 static int mid_groups(int n, int gate) { return gate ? (n + 7) / 8 : (n + 15) / 16; }
 
 // 1 if the skinny kernel takes this product.
@@ -519,7 +526,7 @@ ATOM_EXPORT int atom_gemm_skinny_supports(int m, int n, int k) {
 
 // Into how many slices atom_gemm_skinny cuts K for this product (1: it writes y itself).
 ATOM_EXPORT int atom_gemm_skinny_splits(int m, int n, int k, int gate) {
-  if (m > 16) return mid_plan(mid_groups(n, gate), k).splits;
+  if (takes_mid(m, gate)) return mid_plan(mid_groups(n, gate), k).splits;
   return skinny_plan(max(m, 1), skinny_tiles(n, gate), k).splits;
 }
 
@@ -542,7 +549,7 @@ ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias
   p.halves = m > 64 ? 2 : 1;
   p.rows_half = ((m + p.halves - 1) / p.halves + 15) / 16 * 16;
   const int mt = p.rows_half / 16;
-  if (m > 16) {
+  if (takes_mid(m, gate)) {
     if ((uintptr_t)y & 15) return ATOM_BAD_SHAPE;
     const MidPlan plan = mid_plan(mid_groups(n, gate), k);
     p.tiles = plan.tiles; p.splits = plan.splits; p.kslice = plan.kslice;
@@ -578,6 +585,7 @@ ATOM_EXPORT int atom_gemm_skinny(const void* x, const void* w, const float* bias
     const bool turn = p.splits == 1;
     const bool exact = k % 128 == 0;   // slices are multiples of 1024
     switch (mt) {
+      case 1: GO(1); break;
       case 2: GO(2); break;
       case 3: GO(3); break;
       default: GO(4); break;
