@@ -221,9 +221,8 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(SkinnyParams p) {
 // 16 W rows of w and a range of K; a chunk is 128 k of those rows and of the rows of x.  Each wave loads
 // its own 16 rows of w and a share of the rows of x (the same whole-cache-line loads as above, four
 // chunks in flight a wave) and writes them to one of two LDS buffers; after the block's barrier it
-// multiplies its rows of w with every 16 rows of x.  The more waves, the fewer times x is read; wide
-// products take the W that fills the chip best and are not cut, narrow ones four waves and as many
-// slices of K as it takes to have about 256 blocks.
+// multiplies its rows of w with every 16 rows of x.  The more waves, the fewer times x is read; mid_plan()
+// chooses their number and the slices of K.
 //
 // SiLU-gate: a wave's 16 rows are 8 gate and 8 up rows of the same 8 columns, ordered so that a lane's
 // four results are two gate values and the two up values of the same columns.
