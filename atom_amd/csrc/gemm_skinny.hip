@@ -29,6 +29,9 @@
 // Needs K % 8 == 0 (16-byte loads).  Any N, any M <= 64; atom_gemm_skinny_supports says which products
 // with up to 128 rows it takes.
 #include "common.h"
+#include "linear_static.h"
+
+#include <mutex>
 
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -637,4 +640,60 @@ ATOM_EXPORT int atom_splitk_reduce(const float* partial, const float* bias, void
   else hipLaunchKernelGGL(splitk_reduce_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, partial, bias,
                           (bf16_t*)y, total, n, splits);
   return launch_status();
+}
+
+// ------------------------------------------------------------------ the product that allocates nothing
+//
+// The slices between the product and the reduction live in this array, one copy on every GPU.  In host
+// code its name is only a handle: the address that kernels and copies take is the one that
+// hipGetSymbolAddress returns on the device in question, kept per device in static_slices[].
+static __device__ __align__(256) float scratch[kLinearStaticFloats];
+
+constexpr int kStaticMaxDevices = 64;
+static float* static_slices[kStaticMaxDevices];   // device address of `scratch` on each device, once known
+static std::mutex static_slices_lock;
+
+// The current device's copy of the array, or null with `status` set.
+static float* static_slices_here(int* status) {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kStaticMaxDevices) {
+    *status = ATOM_LAUNCH_FAILED;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(static_slices_lock);
+  if (!static_slices[device]) {
+    float* ptr = nullptr;
+    if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      *status = ATOM_LAUNCH_FAILED;
+      return nullptr;
+    }
+    static_slices[device] = ptr;
+  }
+  *status = ATOM_OK;
+  return static_slices[device];
+}
+
+ATOM_EXPORT int atom_linear_skinny_static_init(void) {
+  int status = ATOM_OK;
+  static_slices_here(&status);
+  return status;
+}
+
+ATOM_EXPORT long atom_linear_skinny_static_limit(void) { return kLinearStaticFloats; }
+
+ATOM_EXPORT int atom_linear_skinny_static(const void* x, const void* w, const float* bias, void* y, int m, int n,
+                                          int k, int out_f32, hipStream_t stream) {
+  if (m < 0 || n <= 0 || k <= 0 || !x || !w || !y) return ATOM_BAD_SHAPE;
+  if (k % 8 || !atom_gemm_skinny_supports(max(m, 1), n, k)) return ATOM_UNSUPPORTED;
+  if (m == 0) return ATOM_OK;
+  const int splits = atom_gemm_skinny_splits(m, n, k, 0);
+  if (splits == 1) return atom_gemm_skinny(x, w, bias, y, nullptr, m, n, k, out_f32, 0, stream);
+  if ((long)splits * m * n > kLinearStaticFloats) return ATOM_TOO_LARGE;
+  int status = ATOM_OK;
+  float* slices = static_slices_here(&status);
+  if (!slices) return status;
+  status = atom_gemm_skinny(x, w, nullptr, nullptr, slices, m, n, k, 0, 0, stream);
+  if (status != ATOM_OK) return status;
+  return atom_splitk_reduce(slices, bias, y, m, n, splits, out_f32, stream);
 }
