@@ -1,10 +1,11 @@
-"""Device memory of the cache: the pages of every run of a layer that keeps keys and
-values, and the state tensors of every run that keeps a per-request state.
+"""Device memory of the cache: what every run of a layer keeps between steps, allocated
+as its cache kind says (``cache.kinds``): pages of keys and values, per-request state,
+or whatever another registered kind holds.
 
 Sizing follows the reference's rule of reserving fixed per-request needs first and
 giving the rest to the pages that grow with context
-(atom/model_ops/attentions/sub_pool_spec.py:203-246): window groups and state are sized
-by ``max_num_seqs``; groups that keep every key get the remaining bytes.
+(atom/model_ops/attentions/sub_pool_spec.py:203-246): window groups and per-slot memory
+are sized by ``max_num_seqs``; groups that keep every key get the remaining bytes.
 """
 
 from __future__ import annotations
@@ -13,8 +14,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..engine.context import KVBinding, StateBinding
-from ..parts.base import KVCacheNeed, StateNeed
+from .kinds import CacheKind, kind_of
 from .manager import GroupSpec
 
 
@@ -23,26 +23,25 @@ class CachePlan:
     groups: list[GroupSpec]
     run_group: list[int | None]   # per run of the order: its group, or None if it keeps no pages
     bytes_per_page: list[int]     # per group, summed over the runs that own pages in it
+    bytes_per_slot: int = 0       # memory of fixed size per request, summed over the runs that own some
 
-    def total_bytes(self) -> int:
-        return sum(g.num_pages * b for g, b in zip(self.groups, self.bytes_per_page))
-
-
-def _elem_size(dtype: torch.dtype) -> int:
-    return torch.empty((), dtype=dtype).element_size()
+    def total_bytes(self, num_slots: int = 0) -> int:
+        return sum(g.num_pages * b for g, b in zip(self.groups, self.bytes_per_page)) + num_slots * self.bytes_per_slot
 
 
 def group_runs(model) -> tuple[list[int | None], list[int | None]]:
-    """(window of each group, group of each run).  Runs whose mixers keep keys with the same
+    """(window of each group, group of each run).  Runs whose mixers keep pages with the same
     window share a group, that is, block tables."""
     windows: list[int | None] = []
     run_group: list[int | None] = []
     for run in model.order:
         need = model.blocks[run.layer].mixer.cache_need()
-        if isinstance(need, KVCacheNeed):
-            if need.window not in windows:
-                windows.append(need.window)
-            run_group.append(windows.index(need.window))
+        kind = kind_of(need)
+        if kind is not None and kind.paged:
+            window = kind.window(need)
+            if window not in windows:
+                windows.append(window)
+            run_group.append(windows.index(window))
         else:
             run_group.append(None)
     return windows, run_group
@@ -54,11 +53,17 @@ def plan_cache(model, page_size: int, dtype: torch.dtype, *, num_pages: int | No
     """Either ``num_pages`` for every group, or a byte budget to divide."""
     windows, run_group = group_runs(model)
     per_page = [0] * len(windows)
+    per_slot = 0
     for run, group in zip(model.order, run_group):
-        if group is None or run.reads_run is not None:
+        if run.reads_run is not None:
             continue
         need = model.blocks[run.layer].mixer.cache_need()
-        per_page[group] += 2 * need.num_kv_heads * need.head_dim * page_size * _elem_size(dtype)
+        kind = kind_of(need)
+        if kind is None:
+            continue
+        per_slot += kind.request_bytes(need, dtype)
+        if group is not None:
+            per_page[group] += kind.page_bytes(need, page_size, dtype)
     if num_pages is not None:
         counts = [num_pages] * len(windows)
     else:
@@ -66,7 +71,7 @@ def plan_cache(model, page_size: int, dtype: torch.dtype, *, num_pages: int | No
             raise ValueError("plan_cache needs num_pages or budget_bytes")
         full_pages = -(-max_model_len // page_size)
         counts = [0] * len(windows)
-        left = budget_bytes
+        left = budget_bytes - per_slot * max_num_seqs
         for gi, w in enumerate(windows):
             if w is None:
                 continue
@@ -79,7 +84,7 @@ def plan_cache(model, page_size: int, dtype: torch.dtype, *, num_pages: int | No
             for gi in full:
                 counts[gi] = pages
     groups = [GroupSpec(page_size, c, w) for c, w in zip(counts, windows)]
-    return CachePlan(groups, run_group, per_page)
+    return CachePlan(groups, run_group, per_page, per_slot)
 
 
 class CacheStorage:
@@ -87,32 +92,39 @@ class CacheStorage:
 
     def __init__(self, model, plan: CachePlan, num_state_slots: int, device, dtype: torch.dtype):
         self.plan = plan
+        self.device = torch.device(device)
         self.bindings: list = []
-        self.state_tensors: list[torch.Tensor] = []
+        self._owned: list[tuple] = []    # (kind, binding) of every run that owns memory
         for i, (run, group) in enumerate(zip(model.order, plan.run_group)):
             need = model.blocks[run.layer].mixer.cache_need()
-            if isinstance(need, KVCacheNeed):
-                if run.reads_run is not None:
-                    src = self.bindings[run.reads_run]
-                    self.bindings.append(KVBinding(src.group, src.k_cache, src.v_cache, writes=False))
-                    continue
-                g = plan.groups[group]
-                k = torch.zeros((g.num_pages, need.num_kv_heads, g.page_size, need.head_dim), dtype=dtype, device=device)
-                v = torch.zeros((g.num_pages, need.num_kv_heads, need.head_dim, g.page_size), dtype=dtype, device=device)
-                self.bindings.append(KVBinding(group, k, v, writes=True))
-            elif isinstance(need, StateNeed):
-                if run.reads_run is not None:
-                    raise ValueError(f"run {i}: a state cannot be read from another run")
-                state = torch.zeros((num_state_slots, *need.shape), dtype=need.dtype, device=device)
-                self.state_tensors.append(state)
-                self.bindings.append(StateBinding(state))
-            else:
+            kind = kind_of(need)
+            if kind is None:
                 self.bindings.append(None)
+                continue
+            if run.reads_run is not None:
+                try:
+                    self.bindings.append(kind.share(self.bindings[run.reads_run]))
+                except ValueError as e:
+                    raise ValueError(f"run {i}: {e}") from None
+                continue
+            g = plan.groups[group] if group is not None else None
+            binding = kind.allocate(need, group=group, num_pages=g.num_pages if g else 0,
+                                    page_size=g.page_size if g else 0, num_slots=num_state_slots, device=device,
+                                    dtype=dtype)
+            self.bindings.append(binding)
+            self._owned.append((kind, binding))
+        # kinds that clear something when a request starts (the others inherit the base's empty method)
+        self._resettable = [(k, b) for k, b in self._owned if type(k).reset is not CacheKind.reset]
+
+    @property
+    def state_tensors(self) -> list[torch.Tensor]:
+        """The per-request state tensors, in running order."""
+        return [b.state for _, b in self._owned if hasattr(b, "state")]
 
     def reset_state(self, slots: list[int]) -> None:
-        """Zeroes the state of slots whose requests start in this step."""
-        if not slots or not self.state_tensors:
+        """Clears the per-request memory of slots whose requests start in this step."""
+        if not slots or not self._resettable:
             return
-        idx = torch.tensor(slots, dtype=torch.long, device=self.state_tensors[0].device)
-        for state in self.state_tensors:
-            state.index_fill_(0, idx, 0)
+        idx = torch.tensor(slots, dtype=torch.long, device=self.device)
+        for kind, binding in self._resettable:
+            kind.reset(binding, idx)

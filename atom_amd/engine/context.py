@@ -1,32 +1,42 @@
-"""What one step hands to the parts: the kernel library, the flat token axis and,
-per group of layers that share block tables, where keys are written and read."""
+"""What one step hands to the parts: the kernel library, the flat token axis and the batch's
+arrays on the device; per group of layers that share block tables, where keys are written and
+read; and whatever each mixer asked for in its ``prepare_step``.
+
+Everything a kernel needs to know about the batch is a device array here, in eager steps and in
+steps replayed from a captured graph alike.  The host-side lists exist only in eager steps."""
 
 from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+import numpy as np
 import torch
 
-from ..kernels.hip import AttentionMeta
+from ..cache.kinds import KVBinding, StateBinding  # noqa: F401  (their home used to be this module)
 
 
 @dataclass
-class KVBinding:
-    """The pages of one run of a layer.  ``writes`` is False for a run that reads the
-    keys and values another run wrote."""
+class BatchView:
+    """A step's batch as a mixer's ``prepare_step`` sees it, on the host.  Requests that bring more
+    than one token (prompt portions) come first on the token axis, the single tokens after them."""
 
-    group: int
-    k_cache: torch.Tensor  # [num_pages, Hkv, page_size, D]
-    v_cache: torch.Tensor  # [num_pages, Hkv, D, page_size]
-    writes: bool = True
+    ops: object
+    dtype: torch.dtype             # the type of the step's activations
+    q_lens: list[int]              # tokens of each request in this step
+    cached: list[int]              # tokens of each request before this step
+    num_prefill: int               # how many requests bring more than one token
+    page_sizes: list[int]          # of each group of layers
+    # the step is (or will be) replayed from a captured graph: rows beyond the live requests are padding
+    # with one token and no context, and the arrays' shapes may depend on ``q_lens`` only
+    replayed: bool = False
 
+    @property
+    def num_seqs(self) -> int:
+        return len(self.q_lens)
 
-@dataclass
-class StateBinding:
-    """The per-request state of one run of a layer: ``state[slot]`` belongs to the request
-    that holds ``slot``; it is zero when the request's first tokens arrive."""
-
-    state: torch.Tensor  # [num_slots, *shape]
+    @property
+    def max_q_len(self) -> int:
+        return max(self.q_lens) if self.q_lens else 0
 
 
 @dataclass
@@ -36,11 +46,35 @@ class StepContext:
     device: torch.device
     num_tokens: int
     num_seqs: int
-    positions: torch.Tensor                      # int32 [T]
-    attention: dict[int, AttentionMeta] = field(default_factory=dict)
-    slot_mappings: dict[int, torch.Tensor] = field(default_factory=dict)  # int32 [T] per group
-    # host-side copies, for mixers that walk requests themselves
-    seq_starts: list[int] = field(default_factory=list)   # first row of each request in the token axis
-    seq_lens: list[int] = field(default_factory=list)     # rows of each request in this step
-    seq_cached: list[int] = field(default_factory=list)   # tokens of each request before this step
-    state_slots: list[int] = field(default_factory=list)  # state slot of each request
+    positions: torch.Tensor                      # int32 [T] absolute position of each token in its request
+    token_seq: torch.Tensor | None = None        # int32 [T] row of its request (-1: padding)
+    cu_seqlens_q: torch.Tensor | None = None     # int32 [S + 1] first token of each request
+    context_lens: torch.Tensor | None = None     # int32 [S] tokens of each request once this step has run
+    cached_lens: torch.Tensor | None = None      # int32 [S] tokens of each request before this step
+    slot_of_seq: torch.Tensor | None = None      # int32 [S] state slot of each request (-1: padding)
+    block_tables: dict[int, torch.Tensor] = field(default_factory=dict)   # per group: int32 [S, width]
+    slot_mappings: dict[int, torch.Tensor] = field(default_factory=dict)  # per group: int32 [T] (-1: no write)
+    page_sizes: dict[int, int] = field(default_factory=dict)
+    # host numbers that pick kernels and grids (upper bounds in a replayed step)
+    num_prefill: int = 0
+    max_q_len: int = 1
+    max_context_len: int = 0
+    replayed: bool = False
+    # what each mixer's ``prepare_step`` returned, on the device: step key -> name -> int32 tensor
+    prepared: dict = field(default_factory=dict)
+    # a scratch dictionary for parts: what one layer derived from the above and the next can use again
+    memo: dict = field(default_factory=dict)
+    # host-side copies, for mixers that walk requests themselves; None in a replayed step
+    seq_starts: list[int] | None = None   # first row of each request in the token axis
+    seq_lens: list[int] | None = None     # rows of each request in this step
+    seq_cached: list[int] | None = None   # tokens of each request before this step
+    state_slots: list[int] | None = None  # state slot of each request
+
+
+def pack_int32(pieces: list[np.ndarray]) -> tuple[list[int], int]:
+    """Offsets of the pieces in one int32 buffer (each padded to 4 ints) and the buffer's length."""
+    offsets, cursor = [], 0
+    for p in pieces:
+        offsets.append(cursor)
+        cursor += (int(p.size) + 3) // 4 * 4
+    return offsets, max(cursor, 4)

@@ -22,10 +22,10 @@ from dataclasses import dataclass, field
 import numpy as np
 import torch
 
+from ..cache.kinds import kind_of
 from ..cache.manager import CacheManager
 from ..cache.storage import CachePlan, CacheStorage
-from ..kernels.hip import AttentionMeta
-from .context import StepContext
+from .context import BatchView, StepContext, pack_int32
 
 
 @dataclass
@@ -48,12 +48,10 @@ class EngineCore:
         self.device = torch.device(device)
         self.dtype = dtype
         self.plan = plan
-        # the prefix cache needs every mixer's memory to be pages that keep all keys
-        from ..parts.base import KVCacheNeed
-
+        # the prefix cache needs every mixer's memory to be pages that keep all that earlier tokens left
         needs = [model.blocks[run.layer].mixer.cache_need() for run in model.order]
         self.prefix_caching = bool(prefix_caching and plan.groups and all(
-            isinstance(n, KVCacheNeed) and n.window is None for n in needs if n is not None))
+            kind_of(n).keeps_every_token(n) for n in needs if n is not None))
         self.manager = CacheManager(plan.groups, max_num_seqs, prefix_caching=self.prefix_caching)
         self.storage = CacheStorage(model, plan, max_num_seqs, self.device, dtype)
         self.lengths: dict[object, int] = {}   # tokens of each live request that are in the cache
@@ -62,6 +60,14 @@ class EngineCore:
         self._fresh_slots: list[int] = []      # slots claimed since the last step: zeroed before it runs
         # where a sampler leaves its tokens when the next step is to read them on the device (StepEntry.feed)
         self.sampled = torch.zeros(max(1, max_num_seqs), dtype=torch.int32, device=self.device)
+        # mixers that want arrays of their own on the device every step, one per distinct step key
+        self.preparers: dict = {}
+        for run in model.order:
+            mixer = model.blocks[run.layer].mixer
+            key = mixer.step_key()
+            if key is not None and key not in self.preparers:
+                self.preparers[key] = mixer
+        self._staging = _Staging(self.device)
         # decode-only steps replay a captured HIP graph per batch-size bucket (None: always eager)
         self.graphs = None
         if graph_sizes:
@@ -177,7 +183,14 @@ class EngineCore:
         if req_id in self.lengths and self.manager.awaited_position(req_id) == position:
             self.manager.amend(req_id, position, token)
 
+    def batch_view(self, q_lens: list[int], cached: list[int], replayed: bool = False) -> BatchView:
+        return BatchView(ops=self.ops, dtype=self.dtype, q_lens=q_lens, cached=cached,
+                         num_prefill=sum(1 for n in q_lens if n > 1),
+                         page_sizes=[g.page_size for g in self.manager.groups], replayed=replayed)
+
     def _build(self, entries: list[StepEntry], order: list[int]):
+        """Every array of the step in one int32 host buffer (pinned), one copy to the device, and the
+        context whose tensors are views of the device buffer."""
         mgr = self.manager
         num_seqs = len(entries)
         q_lens = [len(entries[i].tokens) for i in order]
@@ -189,7 +202,6 @@ class EngineCore:
         tokens = np.empty(total, dtype=np.int32)
         positions = np.empty(total, dtype=np.int32)
         token_seq = np.empty(total, dtype=np.int32)
-        context_lens = np.empty(num_seqs, dtype=np.int32)
         row_of_entry = {}
         for b, i in enumerate(order):
             e = entries[i]
@@ -197,24 +209,12 @@ class EngineCore:
             tokens[s:s + n] = e.tokens
             positions[s:s + n] = np.arange(cached[b], cached[b] + n, dtype=np.int32)
             token_seq[s:s + n] = b
-            context_lens[b] = cached[b] + n
             row_of_entry[i] = s
+        cached_lens = np.asarray(cached, dtype=np.int32)
+        context_lens = cached_lens + np.asarray(q_lens, dtype=np.int32)
+        state_slots = [mgr.state_slot(entries[i].req_id) for i in order]
         want = [row_of_entry[i] + w for i, e in enumerate(entries) for w in e.want]
         want_rows = np.asarray(want, dtype=np.int32)
-
-        # tiles of query rows for the prompt portions (requests with more than one token come
-        # first); the tiles with the most keys are listed first
-        num_prefill = sum(1 for n in q_lens if n > 1)
-        rows_per_tile = 32 if max(q_lens) > 16 else 16
-
-        def tiles_of(rows: int) -> np.ndarray:
-            tile_list = [(b, r0) for b in range(num_prefill) for r0 in range(0, q_lens[b], rows)]
-            tile_list.sort(key=lambda t: -(cached[t[0]] + t[1]))
-            return np.asarray(tile_list, dtype=np.int32).reshape(-1)
-
-        tiles = tiles_of(rows_per_tile)
-        # taller tiles for the prefill kernel whose waves share key tiles (its height depends on the layer)
-        tall = {rows: tiles_of(rows) for rows in (32, 64, 128)} if max(q_lens) >= 32 else {}
 
         feeds = any(e.feed is not None for e in entries)
         feed = np.full(total if feeds else 0, -1, dtype=np.int32)
@@ -222,8 +222,10 @@ class EngineCore:
             for i, e in enumerate(entries):
                 if e.feed is not None:
                     feed[row_of_entry[i]] = e.feed
-        pieces = [tokens, positions, token_seq, starts, context_lens, want_rows, tiles, feed, *tall.values()]
-        group_shapes = []
+        pieces = [tokens, positions, token_seq, starts, context_lens, cached_lens,
+                  np.asarray(state_slots, dtype=np.int32), want_rows, feed]
+        fixed = len(pieces)
+        widths = []
         for gi, g in enumerate(mgr.groups):
             tables = [mgr.block_table(entries[i].req_id, gi) for i in order]
             width = max(1, max(len(t) for t in tables))
@@ -234,40 +236,75 @@ class EngineCore:
             slots = np.concatenate([mgr.slot_mapping(entries[i].req_id, gi, cached[b], q_lens[b])
                                     for b, i in enumerate(order)]) if total else np.empty(0, np.int32)
             pieces += [bt.reshape(-1), slots]
-            group_shapes.append(width)
+            widths.append(width)
+        # what the mixers ask for
+        view = self.batch_view(q_lens, cached)
+        asked = []   # (step key, name, shape, index among the pieces)
+        for key, mixer in self.preparers.items():
+            for name, array in mixer.prepare_step(view).items():
+                array = np.ascontiguousarray(array, dtype=np.int32)
+                asked.append((key, name, array.shape, len(pieces)))
+                pieces.append(array.reshape(-1))
 
-        # one host buffer, one copy; every array is a view of it (each padded to 4 ints)
-        offsets, cursor = [], 0
-        for p in pieces:
-            offsets.append(cursor)
-            cursor += (p.size + 3) // 4 * 4
-        host = np.zeros(max(cursor, 4), dtype=np.int32)
-        for off, p in zip(offsets, pieces):
-            host[off:off + p.size] = p
-        dev = torch.from_numpy(host).to(self.device)
+        offsets, length = pack_int32(pieces)
+        dev = self._staging.send(pieces, offsets, length)
 
-        def view(k):
+        def at(k):
             return dev[offsets[k]:offsets[k] + pieces[k].size]
 
-        d_tokens, d_positions, d_token_seq, d_starts, d_ctx, d_want, d_tiles, d_feed = (view(k) for k in range(8))
+        (d_tokens, d_positions, d_token_seq, d_starts, d_ctx, d_cached, d_slots, d_want, d_feed) = (
+            at(k) for k in range(fixed))
         if feeds:
             self.ops.feed_tokens(d_tokens, d_feed, self.sampled)
-        d_tall = {rows: view(8 + j).view(-1, 2) for j, rows in enumerate(tall)}
-        first_group = 8 + len(tall)
         ctx = StepContext(ops=self.ops, dtype=self.dtype, device=self.device, num_tokens=total, num_seqs=num_seqs,
-                          positions=d_positions, seq_starts=[int(s) for s in starts[:-1]], seq_lens=q_lens,
-                          seq_cached=cached,
-                          state_slots=[mgr.state_slot(entries[i].req_id) for i in order])
+                          positions=d_positions, token_seq=d_token_seq, cu_seqlens_q=d_starts, context_lens=d_ctx,
+                          cached_lens=d_cached, slot_of_seq=d_slots, num_prefill=view.num_prefill,
+                          max_q_len=max(q_lens), max_context_len=int(context_lens.max()),
+                          seq_starts=[int(s) for s in starts[:-1]], seq_lens=q_lens, seq_cached=cached,
+                          state_slots=state_slots)
         for gi, g in enumerate(mgr.groups):
-            bt = view(first_group + 2 * gi).view(num_seqs, group_shapes[gi])
-            ctx.attention[gi] = AttentionMeta(
-                token_seq=d_token_seq, positions=d_positions, block_tables=bt, cu_seqlens_q=d_starts,
-                context_lens=d_ctx, num_seqs=num_seqs, num_tokens=total, max_q_len=max(q_lens),
-                max_context_len=int(context_lens.max()), page_size=g.page_size, num_prefill=num_prefill,
-                prefill_tiles=d_tiles.view(-1, 2) if num_prefill else None, rows_per_tile=rows_per_tile,
-                tiles_by_rows=d_tall or None)
-            ctx.slot_mappings[gi] = view(first_group + 1 + 2 * gi)
+            ctx.block_tables[gi] = at(fixed + 2 * gi).view(num_seqs, widths[gi])
+            ctx.slot_mappings[gi] = at(fixed + 1 + 2 * gi)
+            ctx.page_sizes[gi] = g.page_size
+        for key, name, shape, k in asked:
+            ctx.prepared.setdefault(key, {})[name] = at(k).view(shape)
         return ctx, d_tokens, (d_want if want_rows.size else None)
+
+
+class _Staging:
+    """Pinned host buffers that a step's integer arrays are gathered in before their one copy to the
+    device.  The copy does not block the host; a buffer is written again only after the copy out of it
+    has finished (an event per buffer), the reference's pinned twin with its event
+    (atom/utils/__init__.py:566-617, atom/model_engine/model_runner.py:1356-1401).  Off the GPU: plain memory."""
+
+    def __init__(self, device: torch.device, buffers: int = 3):
+        self.device = device
+        self.pinned = device.type == "cuda"
+        self.hosts: list[torch.Tensor | None] = [None] * buffers
+        self.events = [torch.cuda.Event() if self.pinned else None for _ in range(buffers)]
+        self.pending = [False] * buffers
+        self.turn = 0
+
+    def send(self, pieces: list[np.ndarray], offsets: list[int], length: int) -> torch.Tensor:
+        k = self.turn
+        self.turn = (k + 1) % len(self.hosts)
+        if self.pending[k]:
+            self.events[k].synchronize()
+            self.pending[k] = False
+        host = self.hosts[k]
+        if host is None or host.numel() < length:
+            host = torch.zeros(max(length, 4096) * 2, dtype=torch.int32, pin_memory=self.pinned)
+            self.hosts[k] = host
+        flat = host.numpy()
+        for off, p in zip(offsets, pieces):
+            flat[off:off + p.size] = p
+        if not self.pinned:
+            return host[:length].clone().to(self.device)
+        dev = torch.empty(length, dtype=torch.int32, device=self.device)
+        dev.copy_(host[:length], non_blocking=True)
+        self.events[k].record()
+        self.pending[k] = True
+        return dev
 
 
 TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32, "bf16": torch.bfloat16, "fp32": torch.float32}

@@ -21,7 +21,6 @@ import gc
 import numpy as np
 import torch
 
-from ..kernels.hip import AttentionMeta
 from .context import StepContext
 
 
@@ -70,9 +69,14 @@ class DecodeGraphs:
 
     def _layout(self, size: int) -> tuple[dict[str, tuple[int, int]], int]:
         pieces = [("tokens", size), ("feed", size), ("positions", size), ("token_seq", size), ("starts", size + 1),
-                  ("context_lens", size), ("want", size)]
+                  ("context_lens", size), ("cached_lens", size), ("slot_of_seq", size), ("want", size)]
         for gi, width in enumerate(self.widths):
             pieces += [(f"bt{gi}", size * width), (f"slots{gi}", size)]
+        # what the mixers ask for: in a replayed step the shapes depend on the bucket only
+        view = self.core.batch_view([1] * size, [0] * size, replayed=True)
+        for key, mixer in self.core.preparers.items():
+            for name, array in mixer.prepare_step(view).items():
+                pieces.append((("prepared", key, name, tuple(np.shape(array))), int(np.size(array))))
         offsets, cursor = {}, 0
         for name, n in pieces:
             offsets[name] = (cursor, n)
@@ -100,6 +104,9 @@ class DecodeGraphs:
         token_seq[:] = -1
         ctx_lens = view("context_lens")
         ctx_lens[:] = 0
+        cached_lens, slot_of_seq = view("cached_lens"), view("slot_of_seq")
+        cached_lens[:] = 0
+        slot_of_seq[:] = -1
         view("starts")[:] = np.arange(size + 1, dtype=np.int32)
         view("want")[:] = np.arange(size, dtype=np.int32)
         for b, e in enumerate(entries):
@@ -109,6 +116,8 @@ class DecodeGraphs:
             positions[b] = cached[b]
             token_seq[b] = b
             ctx_lens[b] = cached[b] + 1
+            cached_lens[b] = cached[b]
+            slot_of_seq[b] = mgr.state_slot(e.req_id)
         if not cap.row_state:
             cap.row_state = [[None] * size for _ in self.widths]
         for gi, width in enumerate(self.widths):
@@ -135,6 +144,16 @@ class DecodeGraphs:
                     bt[b, len(table):] = 0
                 state[b] = (serial, len(table))
             # rows beyond the entries keep what they had: their context length is 0, nothing reads them
+        if self.core.preparers:
+            batch = self.core.batch_view([1] * size, list(cached) + [0] * (size - n), replayed=True)
+            for key, mixer in self.core.preparers.items():
+                for name, array in mixer.prepare_step(batch).items():
+                    array = np.ascontiguousarray(array, dtype=np.int32)
+                    piece = ("prepared", key, name, tuple(array.shape))
+                    if piece not in cap.offsets:
+                        raise AssertionError(f"{type(mixer).__name__}.prepare_step: '{name}' has shape {array.shape} "
+                                             f"in this step, not the shape the graph of {size} rows was captured with")
+                    view(piece)[:] = array.reshape(-1)
 
     def _context(self, cap: _Captured):
         core, size = self.core, cap.size
@@ -143,16 +162,21 @@ class DecodeGraphs:
             off, count = cap.offsets[name]
             return cap.dev[off:off + count]
 
+        # every mixer reads the batch from the device; there are no host-side lists in a replayed step
         ctx = StepContext(ops=core.ops, dtype=core.dtype, device=core.device, num_tokens=size, num_seqs=size,
-                          positions=view("positions"), seq_starts=list(range(size)), seq_lens=[1] * size,
-                          seq_cached=[0] * size, state_slots=[0] * size)
+                          positions=view("positions"), token_seq=view("token_seq"), cu_seqlens_q=view("starts"),
+                          context_lens=view("context_lens"), cached_lens=view("cached_lens"),
+                          slot_of_seq=view("slot_of_seq"), num_prefill=0, max_q_len=1,
+                          max_context_len=max(w * g.page_size for w, g in zip(self.widths, core.manager.groups))
+                          if self.widths else self.max_model_len, replayed=True)
         for gi, (g, width) in enumerate(zip(core.manager.groups, self.widths)):
-            ctx.attention[gi] = AttentionMeta(
-                token_seq=view("token_seq"), positions=view("positions"),
-                block_tables=view(f"bt{gi}").view(size, width), cu_seqlens_q=view("starts"),
-                context_lens=view("context_lens"), num_seqs=size, num_tokens=size, max_q_len=1,
-                max_context_len=width * g.page_size, page_size=g.page_size, num_prefill=0, prefill_tiles=None)
+            ctx.block_tables[gi] = view(f"bt{gi}").view(size, width)
             ctx.slot_mappings[gi] = view(f"slots{gi}")
+            ctx.page_sizes[gi] = g.page_size
+        for piece in cap.offsets:
+            if isinstance(piece, tuple) and piece[0] == "prepared":
+                _, key, name, shape = piece
+                ctx.prepared.setdefault(key, {})[name] = view(piece).view(shape)
         return ctx, view("tokens"), view("want"), view("feed")
 
     # ------------------------------------------------------------------ capture and replay

@@ -162,6 +162,18 @@ class HipKernels:
             marked._marked = True
             setattr(self, method, marked)
 
+    def attention_tile_rows(self, dtype, head_dim: int, page_size: int, group: int, max_q_len: int) -> tuple[int, int]:
+        """The heights of the tiles of query rows that ``paged_attention`` wants listed for a step whose
+        longest prompt portion has ``max_q_len`` tokens: (of the kernel whose waves load their own keys, of
+        the kernel whose waves share key tiles); 0 where a kernel is not used (float32 steps list nothing)."""
+        if (dtype != torch.bfloat16 or not self.use_mfma_attention
+                or not self.lib.atom_attention_mfma_supports(head_dim, page_size, group)):
+            return 0, 0
+        tall = 0
+        if max_q_len >= 32 and self.use_tiled_prefill:
+            tall = int(self.lib.atom_attention_prefill_tile_rows(head_dim, page_size, group))
+        return (32 if max_q_len > 16 else 16), tall
+
     def decode_parts(self, seqs: int, hkv: int, max_context: int) -> int:
         """Over how many waves a decode row's keys are split: enough waves to fill the chip,
         at least 64 keys each."""

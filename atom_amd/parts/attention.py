@@ -10,8 +10,10 @@ Norm, rotation and the cache write are one kernel; the scale defaults to
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
+from ..kernels.hip import AttentionMeta
 from .base import MIXERS, POSITION_ENCODINGS, KVCacheNeed, Mixer, ParamSpec, PartChoice
 
 
@@ -68,12 +70,53 @@ class GroupedQueryAttention(Mixer):
                                                       init="one_plus_normal")
         return specs
 
+    # ---- what the attention kernels want to know about a step's batch
+
+    def step_key(self):
+        # the kernels' tile heights depend on the head size and on how many query heads share a KV head
+        return ("attention", self.head_dim, self.num_heads // self.num_kv_heads)
+
+    def _tile_rows(self, ops, dtype, page_size: int, max_q_len: int) -> tuple[int, int]:
+        return ops.attention_tile_rows(dtype, self.head_dim, page_size, self.num_heads // self.num_kv_heads, max_q_len)
+
+    def prepare_step(self, batch) -> dict:
+        """Tiles of query rows of the prompt portions, as (request, first row) pairs, the tiles with the most
+        keys first: one list for every tile height the kernels of this step use."""
+        if not batch.num_prefill:
+            return {}
+        out = {}
+        for page_size in set(batch.page_sizes):
+            for rows in self._tile_rows(batch.ops, batch.dtype, page_size, batch.max_q_len):
+                if rows and f"tiles{rows}" not in out:
+                    tiles = [(b, r0) for b in range(batch.num_prefill) for r0 in range(0, batch.q_lens[b], rows)]
+                    tiles.sort(key=lambda t: -(batch.cached[t[0]] + t[1]))
+                    out[f"tiles{rows}"] = np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
+        return out
+
+    def _meta(self, ctx, group: int) -> AttentionMeta:
+        """The batch as the attention kernels take it, built once a step per group of layers."""
+        key = ("attention meta", self.step_key(), group)
+        meta = ctx.memo.get(key)
+        if meta is None:
+            page_size = ctx.page_sizes[group]
+            arrays = ctx.prepared.get(self.step_key(), {})
+            short, tall = self._tile_rows(ctx.ops, ctx.dtype, page_size, ctx.max_q_len) if ctx.num_prefill else (0, 0)
+            meta = AttentionMeta(
+                token_seq=ctx.token_seq, positions=ctx.positions, block_tables=ctx.block_tables[group],
+                cu_seqlens_q=ctx.cu_seqlens_q, context_lens=ctx.context_lens, num_seqs=ctx.num_seqs,
+                num_tokens=ctx.num_tokens, max_q_len=ctx.max_q_len, max_context_len=ctx.max_context_len,
+                page_size=page_size, num_prefill=ctx.num_prefill,
+                prefill_tiles=arrays.get(f"tiles{short}") if short else None, rows_per_tile=short or 16,
+                tiles_by_rows={tall: arrays[f"tiles{tall}"]} if tall else None)
+            ctx.memo[key] = meta
+        return meta
+
     def forward(self, ctx, x, cache):
         ops = ctx.ops
         tokens = x.shape[0]
         qkv = ops.linear(x, self.params["qkv.weight"], self.p("qkv.bias"), defer=True)
         q = torch.empty((tokens, self.num_heads, self.head_dim), dtype=x.dtype, device=x.device)
-        meta = ctx.attention[cache.group]
+        meta = self._meta(ctx, cache.group)
         rope = self.rope
         ops.qk_norm_rope_kv_write(
             qkv, q, cache.k_cache, cache.v_cache, self.p("q_norm.weight"), self.p("k_norm.weight"),

@@ -144,8 +144,23 @@ class Mixer(Part):
     #: only through device arrays of ``ctx``: a decode step of such mixers may be replayed as a HIP graph
     graph_safe = False
 
-    def cache_need(self) -> KVCacheNeed | StateNeed | None:
+    def cache_need(self):
+        """What this mixer keeps between steps: a ``KVCacheNeed``, a ``StateNeed``, an object of any other
+        registered cache kind (``cache.kinds.register_cache_kind``), or None."""
         return None
+
+    def step_key(self):
+        """Mixers that return equal keys (hashable, not None) share one ``prepare_step`` a step; None:
+        this mixer prepares nothing."""
+        return None
+
+    def prepare_step(self, batch) -> dict:
+        """Integer arrays (numpy int32, any shape) that this mixer's kernels want on the device for this
+        step, by name, derived on the host from ``batch`` (an ``engine.context.BatchView``).  The engine
+        copies them with the step's other arrays in its one transfer and hands them back as device
+        tensors: ``ctx.prepared[self.step_key()][name]``.  For a batch with ``batch.replayed`` set the
+        arrays' shapes may depend on ``batch.q_lens`` only: they live in a captured graph's fixed buffer."""
+        return {}
 
     def forward(self, ctx, x: torch.Tensor, cache) -> torch.Tensor:
         """``cache`` is what the engine bound to this run of the layer: a ``KVBinding`` for a

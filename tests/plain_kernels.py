@@ -74,6 +74,9 @@ class PlainKernels:
                 v_cache[page, :, :, off] = v[i].to(v_cache.dtype)
         return q_out
 
+    def attention_tile_rows(self, dtype, head_dim, page_size, group, max_q_len):
+        return 0, 0   # this attention walks tokens, it wants no tiles listed
+
     def paged_attention(self, q, k_cache, v_cache, out, meta, scale, window=None, parts=None):
         tokens, hq, d = q.shape
         page_size = k_cache.shape[2]

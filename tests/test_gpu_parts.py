@@ -12,11 +12,10 @@ import torch
 
 import plain_model as pm
 from helpers import gpu_ops
-from atom_amd.cache import CacheManager, GroupSpec
+from atom_amd.cache import CacheKind, CacheManager, GroupSpec, kind_of, register_cache_kind, unregister_cache_kind
 from atom_amd.config import ModelConfig, register_architecture, unregister_architecture
-from atom_amd.engine.context import KVBinding, StepContext
+from atom_amd.engine.context import BatchView, KVBinding, StepContext
 from atom_amd.engine.core import StepEntry, build_core, load_model
-from atom_amd.kernels.hip import AttentionMeta
 from atom_amd.models.model import ModelSpec
 from atom_amd.parts import (FEED_FORWARDS, MIXERS, POSITION_ENCODINGS, FeedForward, GatedMLP,
                             GroupedQueryAttention, LMHead, Mixer, ParamSpec, PartChoice, PositionEncoding, PreNormBlock,
@@ -48,8 +47,9 @@ def fill(part, dtype, seed=0, scale=0.3):
     return out
 
 
-def ctx_for(dtype, positions, page_size=16, group=0, num_pages=None):
-    """A one-request step context: the request's tokens at ``positions`` (consecutive)."""
+def ctx_for(dtype, positions, page_size=16, group=0, num_pages=None, mixer=None):
+    """A one-request step context: the request's tokens at ``positions`` (consecutive), with what
+    ``mixer`` asks for in its ``prepare_step``."""
     n = len(positions)
     end = positions[-1] + 1
     num_pages = num_pages or -(-end // page_size) + 2
@@ -58,17 +58,20 @@ def ctx_for(dtype, positions, page_size=16, group=0, num_pages=None):
     mgr.cover("r", 0, end)
     table = torch.tensor([mgr.block_table("r", 0)], dtype=torch.int32, device=DEV)
     pos = torch.tensor(positions, dtype=torch.int32, device=DEV)
-    meta = AttentionMeta(
-        token_seq=torch.zeros(n, dtype=torch.int32, device=DEV), positions=pos, block_tables=table,
-        cu_seqlens_q=torch.tensor([0, n], dtype=torch.int32, device=DEV),
-        context_lens=torch.tensor([end], dtype=torch.int32, device=DEV), num_seqs=1, num_tokens=n, max_q_len=n,
-        max_context_len=end, page_size=page_size, num_prefill=1 if n > 1 else 0,
-        prefill_tiles=torch.tensor([(0, r) for r in range(0, n, 32)], dtype=torch.int32, device=DEV) if n > 1 else None,
-        rows_per_tile=32)
     slots = torch.from_numpy(mgr.slot_mapping("r", 0, positions[0], n)).to(DEV)
-    return StepContext(ops=gpu_ops(), dtype=dtype, device=torch.device(DEV), num_tokens=n, num_seqs=1, positions=pos,
-                       attention={group: meta}, slot_mappings={group: slots}, seq_starts=[0], seq_lens=[n],
-                       seq_cached=[positions[0]], state_slots=[0]), num_pages
+    i32 = lambda values: torch.tensor(values, dtype=torch.int32, device=DEV)  # noqa: E731
+    ctx = StepContext(ops=gpu_ops(), dtype=dtype, device=torch.device(DEV), num_tokens=n, num_seqs=1, positions=pos,
+                      token_seq=torch.zeros(n, dtype=torch.int32, device=DEV), cu_seqlens_q=i32([0, n]),
+                      context_lens=i32([end]), cached_lens=i32([positions[0]]), slot_of_seq=i32([0]),
+                      block_tables={group: table}, slot_mappings={group: slots}, page_sizes={group: page_size},
+                      num_prefill=1 if n > 1 else 0, max_q_len=n, max_context_len=end,
+                      seq_starts=[0], seq_lens=[n], seq_cached=[positions[0]], state_slots=[0])
+    if mixer is not None:   # what the engine does with a mixer's ``prepare_step``: its arrays, on the device
+        view = BatchView(ops=ctx.ops, dtype=dtype, q_lens=[n], cached=[positions[0]], num_prefill=ctx.num_prefill,
+                         page_sizes=[page_size])
+        ctx.prepared[mixer.step_key()] = {name: torch.from_numpy(a).to(DEV)
+                                          for name, a in mixer.prepare_step(view).items()}
+    return ctx, num_pages
 
 
 def check(got, want, dtype):
@@ -118,7 +121,7 @@ def test_attention_part(dtype, hq, hkv, d, bias, window):
                                  position_encoding=rope, prefix="a")
     w = fill(attn, dtype, seed=3, scale=0.2)
     n = 37
-    ctx, pages = ctx_for(dtype, list(range(n)), page_size=8)
+    ctx, pages = ctx_for(dtype, list(range(n)), page_size=8, mixer=attn)
     cache = KVBinding(0, torch.zeros((pages, hkv, 8, d), dtype=dtype, device=DEV),
                       torch.zeros((pages, hkv, d, 8), dtype=dtype, device=DEV))
     x = rnd((n, hidden), 4).to(dtype)
@@ -135,8 +138,8 @@ def test_attention_part(dtype, hq, hkv, d, bias, window):
     check(got, want, dtype)
     # the same tokens in two steps over the cache the first step left
     cache2 = KVBinding(0, torch.zeros_like(cache.k_cache), torch.zeros_like(cache.v_cache))
-    ctx_a, _ = ctx_for(dtype, list(range(20)), page_size=8, num_pages=pages)
-    ctx_b, _ = ctx_for(dtype, list(range(20, n)), page_size=8, num_pages=pages)
+    ctx_a, _ = ctx_for(dtype, list(range(20)), page_size=8, num_pages=pages, mixer=attn)
+    ctx_b, _ = ctx_for(dtype, list(range(20, n)), page_size=8, num_pages=pages, mixer=attn)
     first = attn.forward(ctx_a, x[:20].to(DEV), cache2)
     second = attn.forward(ctx_b, x[20:].to(DEV), cache2)
     check(torch.cat((first, second)), want, dtype)
@@ -182,7 +185,7 @@ def test_prenorm_block(dtype):
         feed_forward=PartChoice("gated_mlp", {"hidden_size": 64, "intermediate_size": 100}), norm=norm, prefix="model.layers.0")
     w = fill(block, dtype, seed=9, scale=0.2)
     n = 21
-    ctx, pages = ctx_for(dtype, list(range(n)))
+    ctx, pages = ctx_for(dtype, list(range(n)), mixer=block.mixer)
     cache = KVBinding(0, torch.zeros((pages, 2, 16, 16), dtype=dtype, device=DEV), torch.zeros((pages, 2, 16, 16), dtype=dtype, device=DEV))
     x, r = rnd((n, 64), 10).to(dtype), rnd((n, 64), 11)
     hidden, res = block.forward(ctx, x.to(DEV), r.to(DEV), cache)
@@ -213,7 +216,11 @@ def test_prenorm_block(dtype):
 
 class RunningMeanMixer(Mixer):
     """y_t = W . mean(x_0 .. x_t): the state of a request is the running sum of its inputs and the
-    number of tokens seen, a fixed size whatever the context."""
+    number of tokens seen, a fixed size whatever the context.  It reads the batch from the step's
+    device arrays only and runs the same operations for every batch, so a decode step with it can be
+    replayed from a captured graph; padding rows (request -1, state slot -1) change no state."""
+
+    graph_safe = True
 
     def __init__(self, hidden_size: int, prefix: str = ""):
         super().__init__(prefix)
@@ -226,14 +233,25 @@ class RunningMeanMixer(Mixer):
         return StateNeed((self.hidden_size + 1,), torch.float32)
 
     def forward(self, ctx, x, cache):
-        out = torch.empty_like(x)
-        for start, n, slot in zip(ctx.seq_starts, ctx.seq_lens, ctx.state_slots):
-            state = cache.state[slot]
-            sums = state[:-1] + torch.cumsum(x[start:start + n].float(), dim=0)
-            counts = state[-1] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
-            out[start:start + n] = (sums / counts[:, None]).to(x.dtype)
-            state[:-1] = sums[-1]
-            state[-1] = counts[-1]
+        state = cache.state                                       # [slots, hidden + 1]
+        seq = ctx.token_seq.long()                                # request of each token, -1 for padding
+        live = (seq >= 0)
+        seq = seq.clamp(min=0)
+        starts = ctx.cu_seqlens_q.long()
+        slot = ctx.slot_of_seq.long()
+        slot_live = (slot >= 0)
+        slot = slot.clamp(min=0)
+        xs = x.double() * live[:, None]
+        running = torch.cumsum(xs, dim=0)                         # over the whole token axis ...
+        before = (running - xs).index_select(0, starts[:-1])      # ... minus what precedes each request's rows
+        old = state.double().index_select(0, slot)                # [S, hidden + 1]
+        sums = old[:, :-1].index_select(0, seq) + running - before.index_select(0, seq)
+        rows = torch.arange(x.shape[0], device=x.device)
+        counts = old[:, -1].index_select(0, seq) + (rows - starts[:-1].index_select(0, seq) + 1)
+        out = (sums / counts[:, None]).to(x.dtype)
+        last = (starts[1:] - 1).clamp(min=0)                      # each request's last row of this step
+        new = torch.cat((sums.index_select(0, last), counts.index_select(0, last)[:, None]), dim=1)
+        state.index_add_(0, slot, ((new - old) * slot_live[:, None]).float())
         return ctx.ops.linear(out, self.params["mix.weight"])
 
 
@@ -310,7 +328,9 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype, tmp_path):
         assert "model.layers.0.self_attn.mix.weight" in tensors and "model.layers.1.self_attn.q_proj.weight" in tensors
         model, loaded = load_model(folder, dtype=dtype, device=DEV)
         assert isinstance(loaded, ToyConfig) and isinstance(model.blocks[0].mixer, RunningMeanMixer)
-        core = build_core(model, gpu_ops(), dtype=dtype, device=DEV, page_size=16, num_pages=12, max_num_seqs=3)
+        core = build_core(model, gpu_ops(), dtype=dtype, device=DEV, page_size=16, num_pages=12, max_num_seqs=3,
+                          graph_sizes=[2])
+        assert core.graphs is not None, "a model whose stateful mixer is graph safe decodes through graphs"
         assert len(core.storage.state_tensors) == 2 and core.storage.state_tensors[0].shape == (3, 41)
         g = torch.Generator().manual_seed(0)
         reqs = {r: torch.randint(0, 97, (n,), generator=g).tolist() for r, n in (("a", 50), ("b", 23), ("c", 70))}
@@ -329,10 +349,16 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype, tmp_path):
         step([("a", 0, 20)])
         step([("a", 20, 21), ("b", 0, 23)])
         core.close("b")                       # b's slot goes back ...
-        step([("a", 21, 50), ("c", 0, 2)])    # ... and c starts in it with a zeroed state
-        step([("c", 2, 3)])
-        step([("c", 3, 70)])
+        step([("a", 21, 40), ("c", 0, 2)])    # ... and c starts in it with a zeroed state
         assert core.manager.state_slot("c") == 1
+        assert core.graphs.replays == 0
+        for t in range(10):                   # both decode: a replayed graph of two rows
+            step([("a", 40 + t, 41 + t), ("c", 2 + t, 3 + t)])
+        core.close("a")
+        step([("c", 12, 13)])                 # one request in the graph of two rows: the other row is padding
+        step([("c", 13, 14)])
+        assert core.graphs.replays == 12
+        step([("c", 14, 70)])
         tol = 3e-5 if dtype == torch.float32 else 4e-2
         for r, ids in reqs.items():
             scale = float(want[r].abs().max())
@@ -342,6 +368,129 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype, tmp_path):
     finally:
         MIXERS.unregister("running_mean")
         unregister_architecture("ToyForCausalLM")
+
+
+# ------------------------------------------------------------------ a kind of memory the framework does not know
+
+
+@dataclass(frozen=True)
+class PreviousTokenNeed:
+    """The last input of every request: neither pages nor a ``StateNeed``."""
+    width: int
+
+
+@dataclass
+class PreviousTokenBinding:
+    last: torch.Tensor     # [slots, width] float32
+    seen: torch.Tensor     # [slots] int32, tokens of the request so far
+
+
+class PreviousTokenKind(CacheKind):
+    def request_bytes(self, need, dtype):
+        return need.width * 4 + 4
+
+    def allocate(self, need, *, group, num_pages, page_size, num_slots, device, dtype):
+        return PreviousTokenBinding(torch.full((num_slots, need.width), 7.0, device=device),   # not zero: reset must clear
+                                    torch.full((num_slots,), 3, dtype=torch.int32, device=device))
+
+    def reset(self, binding, slots):
+        binding.last.index_fill_(0, slots, 0)
+        binding.seen.index_fill_(0, slots, 0)
+
+
+class PreviousTokenMixer(Mixer):
+    """y_t = W (x_t + x_{t-1}), x_{-1} = 0; walks the requests through the step's host-side lists."""
+
+    def __init__(self, hidden_size: int, prefix: str = ""):
+        super().__init__(prefix)
+        self.hidden_size = hidden_size
+
+    def param_specs(self):
+        return {"mix.weight": ParamSpec.single("mix.weight", (self.hidden_size, self.hidden_size))}
+
+    def cache_need(self):
+        return PreviousTokenNeed(self.hidden_size)
+
+    def forward(self, ctx, x, cache):
+        assert isinstance(cache, PreviousTokenBinding)
+        shifted = torch.empty_like(x, dtype=torch.float32)
+        for start, n, cached, slot in zip(ctx.seq_starts, ctx.seq_lens, ctx.seq_cached, ctx.state_slots):
+            assert int(cache.seen[slot]) == cached
+            rows = x[start:start + n].float()
+            shifted[start] = cache.last[slot]
+            shifted[start + 1:start + n] = rows[:-1]
+            cache.last[slot] = rows[-1]
+            cache.seen[slot] += n
+        return ctx.ops.linear((x.float() + shifted).to(x.dtype), self.params["mix.weight"])
+
+
+def previous_token_spec(cfg: ToyConfig) -> ModelSpec:
+    norm = PartChoice("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps})
+    ffn = PartChoice("gated_mlp", {"hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size})
+    blocks = [PartChoice("prenorm", {"mixer": PartChoice("previous_token", {"hidden_size": cfg.hidden_size}),
+                                     "feed_forward": ffn, "norm": norm}) for _ in range(cfg.num_hidden_layers)]
+    return ModelSpec(cfg.vocab_size, cfg.hidden_size, blocks, norm, max_positions=cfg.max_position_embeddings)
+
+
+def plain_previous_token_logits(tensors, cfg: ToyConfig, ids):
+    x = tensors["model.embed_tokens.weight"][torch.tensor(ids)]
+    residual = None
+    for i in range(cfg.num_hidden_layers):
+        p = f"model.layers.{i}."
+        if residual is None:
+            residual, h = x, pm.rms_norm(x, tensors[p + "input_layernorm.weight"], cfg.rms_norm_eps)
+        else:
+            h, residual = pm.add_rms_norm(x, residual, tensors[p + "input_layernorm.weight"], cfg.rms_norm_eps)
+        a = (h + torch.cat((torch.zeros_like(h[:1]), h[:-1]))) @ tensors[p + "self_attn.mix.weight"].T
+        h, residual = pm.add_rms_norm(a, residual, tensors[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps)
+        x = pm.gated_mlp(h, tensors[p + "mlp.gate_proj.weight"], tensors[p + "mlp.up_proj.weight"], tensors[p + "mlp.down_proj.weight"])
+    h, _ = pm.add_rms_norm(x, residual, tensors["model.norm.weight"], cfg.rms_norm_eps)
+    return h @ tensors["lm_head.weight"].T
+
+
+def test_toy_cache_kind_is_registered_planned_and_cleared(tmp_path):
+    """A mixer whose memory is of a kind defined here: the kind is registered, and planning, allocation,
+    clearing for a new request and the step run without a change to the framework's files."""
+    dtype = torch.float32
+    MIXERS.register("previous_token", PreviousTokenMixer)
+    register_cache_kind(PreviousTokenNeed, PreviousTokenKind())
+    register_architecture("PreviousTokenForCausalLM", ToyConfig, previous_token_spec)
+    try:
+        cfg = ToyConfig.from_dict(dict(architectures=["PreviousTokenForCausalLM"], vocab_size=61, hidden_size=24,
+                                       num_hidden_layers=2, max_position_embeddings=64))
+        folder = write_random_model(str(tmp_path / "prev"), cfg, seed=8, std=0.3, norm_std=0.1, dtype=torch.float32)
+        from safetensors.torch import load_file
+        tensors = {k: v.double() for k, v in load_file(folder + "/model.safetensors").items()}
+        model, _ = load_model(folder, dtype=dtype, device=DEV)
+        core = build_core(model, gpu_ops(), dtype=dtype, device=DEV, page_size=16, num_pages=4, max_num_seqs=2)
+        assert core.plan.groups == [] and core.plan.bytes_per_slot == 2 * (24 * 4 + 4)
+        assert all(isinstance(b, PreviousTokenBinding) for b in core.storage.bindings)
+        assert not core.prefix_caching and core.graphs is None
+        g = torch.Generator().manual_seed(3)
+        reqs = {r: torch.randint(0, 61, (n,), generator=g).tolist() for r, n in (("a", 30), ("b", 11), ("c", 9))}
+        got = {r: {} for r in reqs}
+        plan = [[("a", 0, 7)], [("a", 7, 8), ("b", 0, 11)], [("a", 8, 30)], [("c", 0, 1)], [("c", 1, 9)]]
+        for k, parts in enumerate(plan):
+            if k == 3:
+                core.close("b")     # c takes b's slot, which the kind clears
+            logits = core.step([StepEntry(r, reqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in parts])
+            at = 0
+            for r, lo, hi in parts:
+                for pos in range(lo, hi):
+                    got[r][pos] = logits[at].cpu()
+                    at += 1
+        assert core.manager.state_slot("c") == 1
+        for r, ids in reqs.items():
+            want = plain_previous_token_logits(tensors, cfg, ids)
+            scale = float(want.abs().max())
+            for pos in range(len(ids)):
+                assert float((got[r][pos].double() - want[pos]).abs().max()) <= 3e-5 * scale, f"{r} position {pos}"
+        with pytest.raises(KeyError):
+            kind_of(object())
+    finally:
+        MIXERS.unregister("previous_token")
+        unregister_cache_kind(PreviousTokenNeed)
+        unregister_architecture("PreviousTokenForCausalLM")
 
 
 # ------------------------------------------------------------------ toy parts of the other kinds: a feed-forward
