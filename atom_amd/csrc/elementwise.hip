@@ -519,9 +519,10 @@ __global__ void qk_norm_rope_kv_write_kernel(
   T* dst = is_q ? q_out + ((size_t)t * hq + head) * d
                 : k_cache + (((size_t)page * hkv + kv_head) * page_size + off) * (size_t)d;
   const int half = rotary_dim / 2;
-  const int pos = positions[t];
-  const float* cs = cos_table + (size_t)pos * half;
-  const float* sn = sin_table + (size_t)pos * half;
+  // without rotation the three tables may be null: nothing of them is touched then
+  const int pos = half > 0 ? positions[t] : 0;
+  const float* cs = half > 0 ? cos_table + (size_t)pos * half : nullptr;
+  const float* sn = half > 0 ? sin_table + (size_t)pos * half : nullptr;
   for (int j = lane; j < half; j += kWave) {
     float x1 = head_vals[j];
     float x2 = head_vals[j + half];

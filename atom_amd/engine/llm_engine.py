@@ -72,7 +72,9 @@ class _NoEvent:
 
 class LLMEngine:
     def __init__(self, model: str, tokenizer=None, ops=None, weight_source=None, **kwargs):
-        kwargs = {k: v for k, v in kwargs.items() if k in Config.__dataclass_fields__}
+        unknown = sorted(k for k in kwargs if k not in Config.__dataclass_fields__)
+        if unknown:
+            raise TypeError(f"LLMEngine: unknown option(s) {unknown}; known: {sorted(Config.__dataclass_fields__)}")
         self.config = cfg = Config(model, **kwargs)
         self.tokenizer = tokenizer if tokenizer is not None else (
             _load_tokenizer(model) if isinstance(model, str) and os.path.isdir(model) else None)
@@ -100,8 +102,10 @@ class LLMEngine:
             max_num_batched_tokens=cfg.max_num_batched_tokens,
             graph_sizes=None if cfg.enforce_eager else cfg.cudagraph_capture_sizes,
             prefix_caching=cfg.enable_prefix_caching)
+        self._log_capacity()
         if self.core.graphs is not None:   # as the reference's engine does before it serves (engine_core.py:131-138)
-            self.core.graphs.capture_all()
+            captured = self.core.graphs.capture_all()
+            logger.info("captured %d decode graphs for batch sizes %s", captured, self.core.graphs.sizes)
         self.scheduler = Scheduler(cfg, self.core)
         self.sampler = Sampler(ops, cfg.device, cfg.max_num_seqs)
         self.seqs: dict[int, Sequence] = {}
@@ -113,15 +117,54 @@ class LLMEngine:
         self._next_stage = 0
 
     def _cache_budget(self) -> int:
-        """Bytes for the cache: the share of device memory ``gpu_memory_utilization`` allows
-        minus what is in use, with a 2 % margin (atom/model_engine/model_runner.py:1591-1611)."""
+        """Bytes for the cache: the share of device memory ``gpu_memory_utilization`` allows minus what is
+        in use, minus what the decode graphs will take and a 2 % margin
+        (atom/model_engine/model_runner.py:1591-1611, 1737-1749)."""
         dev = torch.device(self.config.device)
         if dev.type != "cuda":
             return 64 << 20
         free, total = torch.cuda.mem_get_info(dev)
         used = total - free
-        budget = int(total * self.config.gpu_memory_utilization) - used - int(total * 0.02)
-        return max(0, min(budget, free))
+        graphs = 0 if self.config.enforce_eager else self._graph_estimate()
+        safety = int(total * 0.02)
+        budget = max(0, min(int(total * self.config.gpu_memory_utilization) - used - graphs - safety, free))
+        logger.info("Memory budget: total_gpu=%.2fGB, free=%.2fGB, utilization=%s, in_use=%.2fGB, "
+                    "cudagraph_est=%.2fGB, safety=%.2fGB, available_for_kv=%.2fGB", total / 2**30, free / 2**30,
+                    self.config.gpu_memory_utilization, used / 2**30, graphs / 2**30, safety / 2**30, budget / 2**30)
+        return budget
+
+    def _graph_estimate(self) -> int:
+        """Bytes the decode graphs' shared pool will hold: every bucket keeps its float32 logits, and the
+        buckets share the memory of one step's activations (what a layer frees during capture the next
+        layer takes again), which the largest bucket sizes; product slices and slack on top."""
+        cfg, spec = self.config, self.model.spec
+        sizes = [s for s in cfg.cudagraph_capture_sizes if s <= cfg.max_num_seqs]
+        if not sizes:
+            return 0
+        widest = max((int(p.shape[0]) for block in self.model.blocks for part in block.walk()
+                      for p in part.params.values() if p.dim() == 2), default=spec.hidden_size)
+        live = max(sizes) * (4 * spec.hidden_size + 8 * widest) * 4
+        return sum(sizes) * spec.vocab_size * 4 + 2 * live + (128 << 20)
+
+    def _log_capacity(self) -> None:
+        """How many requests the pages hold at once, by context length
+        (the reference's table, atom/model_engine/model_runner.py:1751-1781)."""
+        cfg = self.config
+        full = [g for g in self.core.plan.groups if g.window is None]
+        if not full:
+            return
+        pages, page = min(g.num_pages for g in full), full[0].page_size
+        lines = []
+        for pct in (10, 30, 50, 70, 90, 100):
+            ctx = max(1, cfg.max_model_len * pct // 100)
+            per_req = -(-ctx // page)
+            by_pages = pages // per_req
+            most = min(cfg.max_num_seqs, by_pages)
+            bound = "slots" if most == cfg.max_num_seqs < by_pages else "blocks"
+            lines.append(f"  {pct:>3}% ({ctx:>7} tok): {per_req:>6} blk/req -> max_concurrent={most:<5} (bound by {bound})")
+        logger.info("Concurrent capacity vs context length (max_model_len=%d, block_size=%d, max_slots=%d, "
+                    "pool_blocks=%d, cache %.2fGB):\n%s", cfg.max_model_len, page, cfg.max_num_seqs, pages,
+                    self.core.plan.total_bytes(cfg.max_num_seqs) / 2**30, "\n".join(lines))
 
     # ------------------------------------------------------------------ requests
 
@@ -149,6 +192,12 @@ class LLMEngine:
             self.scheduler.add(seq)
             out.append(seq)
         return out
+
+    def abort(self, request_id: int) -> bool:
+        """Ends a waiting or running request early (``request_id``: the ``id`` of a sequence that
+        ``add_request`` returned).  It leaves at the next step with ``finish_reason`` "aborted" and what it
+        has generated so far; its pages and slot go back to the pools.  Returns whether it was found."""
+        return self.scheduler.abort(request_id)
 
     def is_finished(self) -> bool:
         return self.scheduler.is_finished() and self._in_flight is None
@@ -248,6 +297,9 @@ class LLMEngine:
         n = seq.num_completion_tokens
         ttft = seq.first_token_time - seq.arrive_time if seq.first_token_time else 0.0
         tpot = (seq.leave_time - seq.first_token_time) / (n - 1) if n > 1 else 0.0
+        logger.info("Request %s finished with reason %s. Input tokens: %d, output tokens: %d, latency: %.2fs, "
+                    "TTFT: %.3fs, TPOT: %.3fs", seq.id, seq.leave_reason, seq.num_prompt_tokens, n,
+                    seq.leave_time - seq.arrive_time, ttft, tpot)
         return {"text": text, "token_ids": ids, "logprobs": seq.logprobs or None,
                 "latency": seq.leave_time - seq.arrive_time, "finish_reason": seq.leave_reason,
                 "num_tokens_input": seq.num_prompt_tokens, "num_tokens_output": n, "ttft": ttft, "tpot": tpot}

@@ -70,9 +70,11 @@ class ScheduledBatch:
 
 
 class Scheduler:
-    def __init__(self, config, core):
-        """``core`` is the ``EngineCore`` whose cache manager this scheduler takes pages from."""
+    def __init__(self, config, core, clock=time.time):
+        """``core`` is the ``EngineCore`` whose cache manager this scheduler takes pages from; ``clock``
+        tells the time (tests pass their own)."""
         self.core = core
+        self.clock = clock
         self.manager = core.manager
         self.max_num_seqs = config.max_num_seqs
         self.max_num_batched_tokens = config.max_num_batched_tokens
@@ -123,20 +125,27 @@ class Scheduler:
         return None
 
     def _chunked_prefill_size(self, num_new: int, budget_left: int, batched: int) -> int:
-        """Tokens to run this step or 0 to wait (atom/model_engine/scheduler.py:1733-1753)."""
-        chunk = min(num_new, budget_left)
-        if chunk >= num_new:
-            return chunk
-        aligned = chunk - chunk % max(self.block_size, 64)
-        return aligned or (0 if batched else chunk)
+        """How many of a prompt's ``num_new`` outstanding tokens run in this step; 0 means wait.  The rule is
+        the reference's (atom/model_engine/scheduler.py:1733-1753): everything if the budget allows; else
+        the budget rounded down to whole units of ``max(block_size, 64)`` tokens; a remainder smaller than
+        one unit runs only when the step would otherwise be empty."""
+        if num_new <= budget_left:
+            return num_new
+        unit = max(self.block_size, 64)
+        whole_units = (budget_left // unit) * unit
+        if whole_units:
+            return whole_units
+        return budget_left if batched == 0 else 0
 
     def _prefill_chunk_for_budget(self, num_new: int, budget_left: int, batched: int) -> int | None:
-        """atom/model_engine/scheduler.py:1755-1767."""
-        if self.enable_chunked_prefill:
-            return self._chunked_prefill_size(num_new, budget_left, batched) or None
-        if num_new > budget_left and batched > 0:
-            return None
-        return num_new
+        """The same for a new request, or None when it has to wait.  Without chunked prefill a prompt runs
+        whole or not at all; it may exceed the budget only in a step of its own
+        (atom/model_engine/scheduler.py:1755-1767)."""
+        if not self.enable_chunked_prefill:
+            fits = num_new <= budget_left or batched == 0
+            return num_new if fits else None
+        size = self._chunked_prefill_size(num_new, budget_left, batched)
+        return size if size > 0 else None
 
     def _passed_delay(self, now: float) -> bool:
         """atom/model_engine/scheduler.py:2761-2777: hold new prompts until the oldest waiting
@@ -170,7 +179,58 @@ class Scheduler:
 
     # ------------------------------------------------------------------ schedule
 
+    def abort(self, seq_id: int) -> bool:
+        """Marks a waiting or running request as aborted (atom/model_engine/engine_utility.py:219-229): it
+        leaves at the next ``schedule`` with the reason "aborted", its pages and slot given back, whether it
+        had started or not (atom/model_engine/scheduler.py:1195-1197, 2284-2285).  What a step that is
+        still running computes for it is dropped.  Returns whether the request was found."""
+        for seq in list(self.running) + list(self.waiting):
+            if seq.id == seq_id and seq.status in (SequenceStatus.WAITING, SequenceStatus.RUNNING):
+                seq.status = SequenceStatus.ABORTED
+                return True
+        return False
+
+    def _leave_aborted(self, seq: Sequence) -> None:
+        seq.leave_reason = "aborted"
+        seq.leave_time = self.clock()
+        seq.awaits_token = False
+        self.core.close(seq.id)
+        self._rejected.append(seq)
+
+    def _sweep_aborted(self) -> None:
+        for seq in [s for s in self.running if s.status == SequenceStatus.ABORTED]:
+            self.running.remove(seq)
+            if seq.awaits_token:          # the placeholder of a step whose result is dropped
+                seq.token_ids.pop()
+            self._leave_aborted(seq)
+
+    def get_next_batch_info(self) -> tuple[bool, int, int]:
+        """What the next step will mostly be, without scheduling it: (it holds prompt tokens, its tokens,
+        its requests).  The reference's estimate (atom/model_engine/scheduler.py:2724-2759), for steps that
+        hold decode tokens and prompt portions together: running requests decode one token each, the rest
+        of the budget goes to unfinished and then to waiting prompts."""
+        decoding = [s for s in self.running if s.status == SequenceStatus.RUNNING and not s.is_partial_prefill]
+        tokens = reqs = min(len(decoding), self.max_num_seqs, self.max_num_batched_tokens)
+        prompt_tokens = 0
+        pending = [s for s in self.running if s.status == SequenceStatus.RUNNING and s.is_partial_prefill]
+        pending += [s for s in self.waiting if s.status == SequenceStatus.WAITING]
+        for seq in pending:
+            left = self.max_num_batched_tokens - tokens
+            if reqs >= self.max_num_seqs or left <= 0:
+                break
+            want = seq.num_tokens - seq.num_cached_tokens
+            if 0 < self.long_prefill_token_threshold < want:
+                want = self.long_prefill_token_threshold
+            take = self._prefill_chunk_for_budget(want, left, tokens)
+            if not take:
+                break
+            tokens += take
+            prompt_tokens += take
+            reqs += 1
+        return prompt_tokens > 0, tokens, reqs
+
     def schedule(self) -> ScheduledBatch | None:
+        self._sweep_aborted()
         if not self.running and not self.waiting:
             return None
         batch = ScheduledBatch()
@@ -223,20 +283,18 @@ class Scheduler:
             batched += chunk
 
         # ---- new requests, in arrival order
-        now = time.time()
+        now = self.clock()
         while (self.waiting and len(batch.items) < self.max_num_seqs and batched < self.max_num_batched_tokens
                and self._passed_delay(now)):
             seq = self.waiting.popleft()
             if seq.status == SequenceStatus.ABORTED:
-                seq.leave_reason = "aborted"
-                seq.leave_time = time.time()
-                self._rejected.append(seq)
+                self._leave_aborted(seq)
                 continue
             reason = self._unschedulable_reason(seq)
             if reason is not None:
                 seq.status = SequenceStatus.FINISHED
                 seq.leave_reason = f"unschedulable: {reason}"
-                seq.leave_time = time.time()
+                seq.leave_time = self.clock()
                 self._rejected.append(seq)
                 continue
             if len(self.running) >= self.max_num_seqs or not mgr.can_open():
@@ -339,7 +397,7 @@ class Scheduler:
         """``sampled`` maps sequence id -> sampled token for every final item.  Returns the
         sequences that finished."""
         finished = []
-        now = time.time()
+        now = self.clock()
         if batch.num_prefill:
             self._last_prompt_latency = step_seconds
         for it in batch.items:

@@ -118,8 +118,8 @@ class HipKernels:
                    "atom_attention_prefill_tile_rows"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
-        # bfloat16 products of few rows run this library's own weight-streaming kernel.  It takes up to 64
-        # rows; beyond 16 (one matrix-core tile of rows) the BLAS library's kernels are faster on gfx950.
+        # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
+        # up to 128 for the narrow products that atom_gemm_skinny_supports names; the BLAS library takes the rest.
         self.use_skinny_gemm = True
         self.skinny_max_rows = 128
         self.use_mfma_attention = True
@@ -430,10 +430,14 @@ class HipKernels:
             result = DeferredSum(partial, bias, out_dtype)
             return result if defer else self.materialize(result)
         if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and self.allow_library_gemm:
-            y = torch.nn.functional.linear(x, weight)
+            if bias is None and out_dtype == torch.bfloat16:
+                return torch.nn.functional.linear(x, weight)
+            # float32 out, or a bias: the library writes its float32 sums as they are, so that logits have the
+            # same precision whatever the number of rows, and a bias is added before anything is rounded
+            y = torch.mm(x, weight.t(), out_dtype=torch.float32)
             if bias is not None:
-                y = (y.float() + bias)
-            return y.to(out_dtype)
+                y += bias
+            return y if out_dtype == torch.float32 else y.to(out_dtype)
         y = torch.empty((m, n), dtype=out_dtype, device=x.device)
         self._done("gemm_f32", self.lib.atom_gemm_f32(
             _ptr(x), self._code(x), _ptr(weight), self._code(weight), _ptr(bias), _ptr(y), self._code(y), m, n, k,

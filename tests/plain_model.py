@@ -194,7 +194,7 @@ def _sub(tensors: dict, prefix: str) -> dict:
     return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def qwen3_logits(cfg: dict, tensors: dict, ids, order=None, dtype=torch.float64) -> torch.Tensor:
+def qwen3_logits(cfg: dict, tensors: dict, ids, order=None, dtype=torch.float64, first_position: int = 0) -> torch.Tensor:
     """Logits [T, V] of one whole sequence.
 
     atom/models/qwen3.py:297-310: embedding; layer 0 norms the embedding and keeps
@@ -206,11 +206,12 @@ def qwen3_logits(cfg: dict, tensors: dict, ids, order=None, dtype=torch.float64)
     ``order`` is the list of layer runs: ``(layer, source)`` pairs where ``source``
     is None for a run that writes keys and values of its own, or the index of an
     earlier run whose keys and values this one reads.  Default: each layer once.
+    ``first_position`` numbers the tokens from there on instead of 0 (for tests of what positions mean).
     """
     cfg = normalise_config(cfg)
     ids = torch.as_tensor(ids, dtype=torch.long)
     tensors = {k: v.to(dtype) for k, v in tensors.items()}
-    positions = torch.arange(ids.numel())
+    positions = torch.arange(ids.numel()) + first_position
     eps = cfg["rms_norm_eps"]
     if order is None:
         order = [(i, None) for i in range(cfg["num_hidden_layers"])]

@@ -210,3 +210,95 @@ def test_steps_launched_ahead_under_random_load(seed):
     reasons = [reason for _, reason in ahead.values()]
     assert any(r.startswith("stop_") or r == "eos" for r in reasons) and "max_tokens" in reasons
     assert llm.scheduler.total_preemptions > 0 and llm.core.manager.pools[0].hits > 0
+
+
+# ------------------------------------------------------------------ options of the entry point
+
+
+def test_unknown_engine_option_is_an_error():
+    from atom_amd import LLMEngine
+    from helpers import tiny_folder
+
+    with pytest.raises(TypeError, match="max_num_seq"):
+        LLMEngine(tiny_folder("A"), dtype="fp32", ops=PlainKernels(), device="cpu", max_num_seq=4)
+
+
+def test_n_samples_fan_out():
+    """``n`` sequences of one prompt (atom/model_engine/llm_engine.py:584-720): distinct seeds give distinct
+    continuations at a temperature, the same as separate requests with those seeds give; greedy gives n equal
+    ones; the later sequences find the prompt's full pages in the prefix cache."""
+    from atom_amd import SamplingParams
+
+    prompt = random_ids("B", 35, 3)
+    llm = _engine(True, enable_prefix_caching=True, max_num_batched_tokens=40)
+    outs = llm.generate([prompt], SamplingParams(temperature=0.9, max_tokens=10, ignore_eos=True, seed=11, n=3))
+    assert len(outs) == 3
+    texts = [tuple(o["token_ids"]) for o in outs]
+    assert len(set(texts)) == 3, "three seeds, three continuations"
+    _idle(llm)
+    hits = llm.core.manager.pools[0].hits
+    assert hits >= 4, "the second and third sequence take the prompt's pages from the prefix cache"
+    singles = _engine(True)
+    for k, want in enumerate(texts):
+        got = singles.generate([prompt], SamplingParams(temperature=0.9, max_tokens=10, ignore_eos=True, seed=11 + k))
+        assert tuple(got[0]["token_ids"]) == want
+    same = llm.generate([prompt], SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True, n=2))
+    assert same[0]["token_ids"] == same[1]["token_ids"]
+
+
+class _WordTokenizer:
+    """Token k is the text "wk "."""
+
+    def encode(self, text, add_special_tokens=True):
+        return [int(w[1:]) for w in text.split()]
+
+    def decode(self, ids):
+        return "".join(f"w{t} " for t in ids)
+
+
+def test_stop_strings_end_a_request():
+    """atom/model_engine/llm_engine.py:661-671, scheduler.py:2296-2312: a stop string is a token sequence;
+    a request ends when its output ends in one."""
+    from atom_amd import LLMEngine, SamplingParams
+    from helpers import tiny_folder
+    from tiny import PAGE
+
+    def make():
+        return LLMEngine(tiny_folder("B"), tokenizer=_WordTokenizer(), dtype="fp32", ops=PlainKernels(), device="cpu",
+                         kv_cache_block_size=PAGE["B"], num_kvcache_blocks=64, max_num_seqs=4)
+
+    prompt = "w5 w17 w200 w3 w9"
+    free = make().generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))[0]
+    ids = free["token_ids"]
+    assert len(ids) == 12 and free["text"] == "".join(f"w{t} " for t in ids)
+    stop = f"w{ids[5]} w{ids[6]}"
+    first = next(k for k in range(1, 12) if ids[k - 1:k + 1] == ids[5:7])
+    out = make().generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True,
+                                                   stop_strings=[stop, "w310 w310"]))[0]
+    assert out["finish_reason"] == "stop_sequence"
+    assert out["token_ids"] == ids[:first + 1]
+
+
+def test_abort_through_the_engine():
+    from atom_amd import SamplingParams
+
+    llm = _engine(True, max_num_seqs=2)    # the third request waits
+    sp = SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=True)
+    keep = llm.add_request(random_ids("B", 12, 1), sp)[0]
+    gone = llm.add_request(random_ids("B", 20, 2), sp)[0]
+    never = llm.add_request(random_ids("B", 9, 3), sp)[0]
+    finished = []
+    for _ in range(6):
+        finished += llm.step()
+    assert gone.num_completion_tokens >= 3
+    assert llm.abort(gone.id) and llm.abort(never.id) is True
+    while not llm.is_finished():
+        finished += llm.step()
+    reasons = {s.id: s.leave_reason for s in finished}
+    assert reasons == {keep.id: "max_tokens", gone.id: "aborted", never.id: "aborted"}
+    assert 3 <= gone.num_completion_tokens < 30 and not gone.awaits_token and never.num_completion_tokens == 0
+    assert keep.num_completion_tokens == 30
+    # the request that stayed is not disturbed: the same tokens as alone
+    alone = _engine(True).generate([keep.token_ids[:12]], sp)[0]
+    assert alone["token_ids"] == keep.completion_token_ids
+    _idle(llm)

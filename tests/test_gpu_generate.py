@@ -39,9 +39,10 @@ def check_greedy(which, dtype, prompts, outs):
             ids.append(token)
 
 
-@pytest.mark.parametrize("which,dtype", [("A", "fp32"), ("B", "fp32"), ("B", "bf16"), ("C", "fp32"), ("C", "bf16")])
+@pytest.mark.parametrize("which,dtype", [("A", "fp32"), ("B", "fp32"), ("B", "bf16"), ("C", "fp32"), ("C", "bf16"),
+                                         ("D", "fp32"), ("D", "bf16")])
 def test_greedy_generation_matches_plain(which, dtype):
-    lens = {"A": (5, 17, 33), "B": (1, 9, 40, 71), "C": (3, 50, 120)}[which]
+    lens = {"A": (5, 17, 33), "B": (1, 9, 40, 71), "C": (3, 50, 120), "D": (4, 70, 300)}[which]
     prompts = [random_ids(which, n, 40 + n) for n in lens]
     llm = engine(which, dtype, max_num_batched_tokens=16 if which == "B" else 64)
     outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8 if which == "A" else 12, ignore_eos=True))
@@ -277,3 +278,30 @@ def test_prefix_cache_reuses_pages_and_changes_nothing(which, dtype):
 def test_prefix_cache_is_off_where_a_window_gives_pages_back():
     llm = engine("C", "fp32", enable_prefix_caching=True)
     assert not llm.core.prefix_caching
+
+
+def test_default_cache_sizing_fills_the_allowed_memory_and_generates():
+    """``num_kvcache_blocks=-1`` (the default): the pool takes what ``gpu_memory_utilization`` leaves after the
+    weights, the decode graphs and a margin (atom/model_engine/model_runner.py:1591-1611); graphs are
+    captured; generation matches the plain implementation."""
+    import torch
+
+    torch.cuda.empty_cache()
+    free, total = torch.cuda.mem_get_info()
+    want_pool = 4 << 30
+    util = min(1.0, (total - free + int(total * 0.02) + want_pool + (1 << 30)) / total)
+    llm = LLMEngine(tiny_folder("D"), dtype="bf16", ops=gpu_ops(), gpu_memory_utilization=util, max_num_seqs=8,
+                    max_model_len=512, cudagraph_capture_sizes=[1, 2, 4, 8])
+    plan = llm.core.plan
+    assert llm.config.num_kvcache_blocks == -1 and llm.config.kv_cache_block_size == 16
+    assert plan.groups[0].num_pages > 8 * 512 // 16, "the pool must hold more than every slot's longest request"
+    assert 0.7 * want_pool <= plan.total_bytes() <= want_pool + (1 << 30)
+    free_after, _ = torch.cuda.mem_get_info()
+    assert total - free_after <= util * total, "weights, cache and graphs stay inside the allowed share"
+    assert llm.core.graphs is not None and sorted(llm.core.graphs.captured) == [1, 2, 4, 8]
+    prompts = [random_ids("D", n, 60 + n) for n in (5, 90, 33)]
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))
+    assert llm.core.graphs.replays > 0
+    check_greedy("D", "bf16", prompts, outs)
+    del llm
+    torch.cuda.empty_cache()

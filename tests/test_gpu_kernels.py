@@ -123,6 +123,28 @@ def test_linear_bf16_library_path():
     assert y32.dtype == torch.float32
 
 
+def test_float32_logits_keep_their_precision_with_many_rows():
+    """A head's float32 output is the float32 sum whatever the number of rows (few rows: the engine's own
+    kernel, many: the library's), so a request's logits do not lose bits when it decodes beside many others;
+    and a bias is added before the product is rounded to bfloat16."""
+    ops = gpu_ops()
+    x, w = rnd((150, 264), torch.bfloat16, 21), rnd((5001, 264), torch.bfloat16, 22, 0.05)
+    want = x.double() @ w.double().T
+    scale = float(want.abs().max())
+    many = ops.linear(x.to(DEV), w.to(DEV), None, out_dtype=torch.float32)
+    assert not ops._skinny(x.to(DEV), w.to(DEV))
+    assert float((many.cpu().double() - want).abs().max()) <= 2e-6 * scale
+    for row in (0, 77, 149):
+        alone = ops.linear(x[row:row + 1].to(DEV).contiguous(), w.to(DEV), None, out_dtype=torch.float32)
+        assert float((alone[0] - many[row]).abs().max()) <= 2e-6 * scale
+    b = rnd((5001,), torch.float32, 23, 2.0)
+    y = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV))
+    exact = (want + b.double()).float().to(torch.bfloat16)      # one rounding of the exact sum
+    off = (y.cpu().float() - exact.float()).abs()
+    assert float((off / exact.float().abs().clamp(min=1e-3)).max()) <= 2.0 ** -7, "at most one bfloat16 step off"
+    assert float((off > 0).float().mean()) < 0.02, "only sums that lie at a rounding boundary may differ"
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hq,hkv,d,rot,page", [(4, 2, 16, 16, 16), (6, 3, 32, 32, 8), (5, 5, 48, 24, 4),
                                               (8, 1, 128, 128, 32), (3, 1, 80, 0, 16), (5, 2, 64, 64, 16),

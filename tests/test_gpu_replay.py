@@ -12,7 +12,8 @@ from tiny import CONFIGS
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [5, 17, 33, 100, 128, 64], "B": [1, 9, 40, 71, 200, 256, 130], "C": [3, 50, 600, 320, 95, 31, 257, 1000]}
+LENGTHS = {"A": [5, 17, 33, 100, 128, 64], "B": [1, 9, 40, 71, 200, 256, 130], "C": [3, 50, 600, 320, 95, 31, 257, 1000],
+           "D": [2, 70, 700, 129, 33, 400]}
 
 
 def _requests(which, seed=0):
@@ -31,7 +32,7 @@ def _oracle(which, requests):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
 def test_cuts_match_plain(which, cut, dtype):
     requests = _requests(which)
@@ -74,7 +75,7 @@ def test_float32_cuts_agree_closely(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "C"])
+@pytest.mark.parametrize("which", ["A", "C", "D"])
 def test_trace_run_program(which, dtype, tmp_path):
     """``bin/trace_run`` itself: mixed trace, pool sized by --max-tokens, logits read from files."""
     requests = _requests(which, seed=1)

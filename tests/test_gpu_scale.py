@@ -193,3 +193,35 @@ def test_pages_far_into_a_large_cache():
     for a, b in zip(low, high):
         assert torch.isfinite(a.float()).all() and torch.equal(a, b)
     assert float(low[0].float().abs().max()) > 0 and float(low[1].float().abs().max()) > 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_serving_layer_sizes_against_the_plain_implementation(dtype, tmp_path_factory):
+    """Two layers of the full layer shape (hidden 4096, 32/8 heads of 128, 12288 wide; a small vocabulary so
+    that the plain implementation's head stays cheap) written as a model folder, run by the engine (most of a
+    500-token prompt in one step, the last tokens one by one) and by the plain implementation on the CPU in
+    float64, which reads the same folder."""
+    import plain_model
+    from atom_amd.engine.core import TORCH_DTYPES, load_model
+    from atom_amd.weights import write_random_model
+
+    folder = getattr(test_serving_layer_sizes_against_the_plain_implementation, "folder", None)
+    if folder is None:
+        cfg = model_config_from_dict({**SHAPE, "vocab_size": 8209})
+        folder = write_random_model(str(tmp_path_factory.mktemp("layers8b") / "m"), cfg, 9, 0.02, 0.1, torch.bfloat16)
+        test_serving_layer_sizes_against_the_plain_implementation.folder = folder
+        plain_cfg, tensors = plain_model.load_folder(folder)
+        ids = torch.randint(0, 8209, (500,), generator=torch.Generator().manual_seed(3)).tolist()
+        test_serving_layer_sizes_against_the_plain_implementation.ids = ids
+        test_serving_layer_sizes_against_the_plain_implementation.want = plain_model.qwen3_logits(plain_cfg, tensors, ids)[-LAST:]
+        del tensors
+    ids = test_serving_layer_sizes_against_the_plain_implementation.ids
+    want = test_serving_layer_sizes_against_the_plain_implementation.want
+    model, _ = load_model(folder, dtype=TORCH_DTYPES[dtype], device="cuda:0")
+    core = build_core(model, gpu_ops(), dtype=TORCH_DTYPES[dtype], device="cuda:0", page_size=16, num_pages=64,
+                      max_num_seqs=2, max_model_len=1024, graph_sizes=[1])
+    head = len(ids) - LAST // 2
+    first = core.step([StepEntry("x", ids[:head], list(range(len(ids) - LAST, head)))]).cpu()
+    rows = [first] + [core.step([StepEntry("x", [tok], [0])]).cpu() for tok in ids[head:]]
+    assert core.graphs.replays == LAST // 2
+    _close(torch.cat(rows), want, dtype, f"{dtype} engine against the plain implementation")

@@ -169,7 +169,7 @@ def test_mlp_is_silu_gate_times_up():
 # ------------------------------------------------------------------ whole model
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_model_is_causal(which):
     cfg, tensors = oracle_weights(which)
     ids = random_ids(which, 40, 3)
@@ -204,6 +204,96 @@ def test_model_attention_block_is_its_parts_in_order():
     assert torch.allclose(got, want, atol=1e-9)
     qr = F.rms_norm(pm.rope_neox(q, cos, sin), (d,), w["q_norm.weight"], cfg["rms_norm_eps"])
     assert not torch.allclose(qr, qn, atol=1e-3), "norm after rotation is a different function here"
+
+
+# The assembly of the parts (what feeds what, where the residual stream starts and where norms sit) is pinned by
+# three reductions to library routines and one invariant, each of which a plausible other arrangement fails.
+
+
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+def test_model_without_attention_is_a_stack_of_library_mlps(which):
+    """With every o_proj zero the mixers add nothing, and what is left is: the residual stream starts as the
+    embedding itself (not its norm); each layer adds MLP(norm(stream)) with the post-attention norm's weight;
+    the final norm sees the sum (atom/models/qwen3.py:248-258, 310).  Written with library routines only."""
+    cfg, tensors = oracle_weights(which)
+    ids = random_ids(which, 9, 21)
+    silent = {k: (torch.zeros_like(v) if k.endswith("o_proj.weight") else v) for k, v in tensors.items()}
+    got = pm.qwen3_logits(cfg, silent, ids)
+    eps = cfg["rms_norm_eps"]
+    hidden = cfg["hidden_size"]
+    head = tensors["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else tensors["lm_head.weight"]
+
+    def stack(stream, norm_of_layer):
+        for layer in range(cfg["num_hidden_layers"]):
+            p = f"model.layers.{layer}."
+            h = F.rms_norm(stream, (hidden,), tensors[p + norm_of_layer], eps)
+            act = F.silu(F.linear(h, tensors[p + "mlp.gate_proj.weight"])) * F.linear(h, tensors[p + "mlp.up_proj.weight"])
+            stream = stream + F.linear(act, tensors[p + "mlp.down_proj.weight"])
+        return F.linear(F.rms_norm(stream, (hidden,), tensors["model.norm.weight"], eps), head)
+
+    embedded = tensors["model.embed_tokens.weight"][torch.tensor(ids)]
+    want = stack(embedded, "post_attention_layernorm.weight")
+    scale = float(want.abs().max())
+    assert torch.allclose(got, want, atol=1e-9 * scale + 1e-12)
+    # arrangements that this rules out: the MLP behind the input norm; a stream that starts from the normed embedding
+    assert float((stack(embedded, "input_layernorm.weight") - got).abs().max()) > 1e-3 * scale
+    normed = F.rms_norm(embedded, (hidden,), tensors["model.layers.0.input_layernorm.weight"], eps)
+    assert float((stack(normed, "post_attention_layernorm.weight") - got).abs().max()) > 1e-3 * scale
+
+
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+def test_model_first_token_goes_through_values_only(which):
+    """One token sees one key, so attention returns its value whatever queries and keys are: with the MLPs
+    silenced (down_proj zero), each layer adds o_proj(v_proj(norm(stream))) with the input norm's weight, the
+    value of KV head ``h // group`` under query head h, neither normed per head nor rotated
+    (atom/models/qwen3.py:146-162)."""
+    cfg, tensors = oracle_weights(which)
+    token = random_ids(which, 1, 5)
+    silent = {k: (torch.zeros_like(v) if k.endswith("down_proj.weight") else v) for k, v in tensors.items()}
+    got = pm.qwen3_logits(cfg, silent, token)
+    eps, hidden = cfg["rms_norm_eps"], cfg["hidden_size"]
+    hq, hkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    stream = tensors["model.embed_tokens.weight"][torch.tensor(token)]
+    for layer in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{layer}."
+        h = F.rms_norm(stream, (hidden,), tensors[p + "input_layernorm.weight"], eps)
+        v = F.linear(h, tensors[p + "self_attn.v_proj.weight"], tensors.get(p + "self_attn.v_proj.bias"))
+        per_head = v.view(1, hkv, d).repeat_interleave(hq // hkv, dim=1)      # consecutive query heads share a KV head
+        stream = stream + F.linear(per_head.reshape(1, hq * d), tensors[p + "self_attn.o_proj.weight"])
+    head = tensors["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else tensors["lm_head.weight"]
+    want = F.linear(F.rms_norm(stream, (hidden,), tensors["model.norm.weight"], eps), head)
+    assert torch.allclose(got, want, atol=1e-9 * float(want.abs().max()) + 1e-12)
+
+
+@pytest.mark.parametrize("which", ["A", "B", "D"])
+def test_model_sees_positions_as_distances_only(which):
+    """Numbering the tokens from 37 instead of 0 changes no logit (beyond the float32 angles): the rotation is
+    the last thing that happens to queries and keys.  A per-head norm *after* the rotation, with weights that
+    differ over the head dimension as they do here, would break this; so would rotating the values."""
+    cfg, tensors = oracle_weights(which)
+    ids = random_ids(which, 30, 8)
+    base = pm.qwen3_logits(cfg, tensors, ids)
+    moved = pm.qwen3_logits(cfg, tensors, ids, first_position=37)
+    scale = float(base.abs().max())
+    assert float((base - moved).abs().max()) <= 2e-4 * scale
+    # the other order is not invariant: the same check on one attention layer with the norm after the rotation
+    w = {k[len("model.layers.0.self_attn."):]: v for k, v in tensors.items() if k.startswith("model.layers.0.self_attn.")}
+    hq, hkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    x = t(12, cfg["hidden_size"], seed=3)
+
+    def norm_after_rotation(first):
+        pos = torch.arange(12) + first
+        cos, sin = pm.rope_angles(pos, d, cfg["rope_theta"])
+        q = F.rms_norm(pm.rope_neox(F.linear(x, w["q_proj.weight"]).view(12, hq, d), cos, sin), (d,), w["q_norm.weight"], 1e-6)
+        k = F.rms_norm(pm.rope_neox(F.linear(x, w["k_proj.weight"]).view(12, hkv, d), cos, sin), (d,), w["k_norm.weight"], 1e-6)
+        return pm.causal_attention(q, k, F.linear(x, w["v_proj.weight"]).view(12, hkv, d), d ** -0.5)
+
+    other = norm_after_rotation(0)
+    assert float((other - norm_after_rotation(37)).abs().max()) > 1e-3 * float(other.abs().max())
+    pos0, pos37 = torch.arange(12), torch.arange(12) + 37
+    a0, _ = pm.self_attention(x, pos0, w, cfg)
+    a37, _ = pm.self_attention(x, pos37, w, cfg)
+    assert float((a0 - a37).abs().max()) <= 2e-4 * float(a0.abs().max())
 
 
 def test_model_head_is_tied_or_not():

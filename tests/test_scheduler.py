@@ -425,3 +425,98 @@ def test_schedule_ahead_declines_and_changes_nothing():
     sched.add(seq(range(100)))
     running = sched.schedule()
     assert not running.items[0].is_final and sched.schedule_ahead(running) is None
+
+
+# ------------------------------------------------------------------ the delay factor, abort, the next batch
+
+
+class FakeClock:
+    def __init__(self):
+        self.now = 1000.0
+
+    def __call__(self):
+        return self.now
+
+
+def test_delay_factor_holds_new_prompts_while_requests_run():
+    """atom/model_engine/scheduler.py:2761-2777: with requests running, a waiting prompt is admitted only
+    once the oldest waiting request has waited longer than delay_factor times the last prompt step's
+    latency; with nothing running it is admitted at once."""
+    clock = FakeClock()
+    sched, _ = make(scheduler_delay_factor=2.0)
+    sched.clock = clock
+    first = seq(range(10), max_tokens=50, ignore_eos=True)
+    first.arrive_time = clock.now
+    sched.add(first)
+    batch = sched.schedule()                      # nothing runs: admitted whatever the delay says
+    assert [it.seq for it in batch.items] == [first]
+    sched.postprocess(batch, {first.id: 5}, step_seconds=0.5)    # the last prompt step took 0.5 s
+    late = seq(range(20, 30), max_tokens=5, ignore_eos=True)
+    late.arrive_time = clock.now
+    sched.add(late)
+    clock.now += 0.9                              # waited 0.9 s <= 2.0 * 0.5 s
+    batch = sched.schedule()
+    assert [it.seq for it in batch.items] == [first] and batch.items[0].is_decode
+    sched.postprocess(batch, {first.id: 5}, step_seconds=0.01)   # a decode step does not change the latency
+    clock.now += 0.2                              # 1.1 s > 1.0 s
+    batch = sched.schedule()
+    assert [it.seq for it in batch.items] == [first, late]
+    # without a delay factor the prompt would have gone in at once
+    sched0, _ = make()
+    a, b = seq(range(10), max_tokens=50, ignore_eos=True), seq(range(20, 30), max_tokens=5, ignore_eos=True)
+    sched0.add(a)
+    run(sched0, sched0.schedule())
+    sched0.add(b)
+    assert [it.seq for it in sched0.schedule().items] == [a, b]
+
+
+def test_abort_of_waiting_and_running_requests_frees_pages():
+    """atom/model_engine/scheduler.py:1195-1197, 2284-2285; engine_utility.py:219-229."""
+    sched, core = make(blocks=20, block=4, max_num_seqs=2)
+    a, b, c = (seq(range(k, k + 9), max_tokens=30, ignore_eos=True) for k in (0, 100, 200))
+    sched.extend([a, b, c])
+    run(sched, sched.schedule())                  # a and b run, c waits (two slots)
+    assert a.status == b.status == SequenceStatus.RUNNING and c.status == SequenceStatus.WAITING
+    used = core.manager.pools[0].num_pages - core.manager.pools[0].num_free
+    assert used == 6
+    assert sched.abort(c.id) and sched.abort(a.id) and not sched.abort(10 ** 9)
+    assert not sched.abort(a.id), "a request is aborted once"
+    batch = sched.schedule()
+    gone = sched.take_rejected()
+    assert {s.id for s in gone} == {a.id, c.id}
+    assert all(s.leave_reason == "aborted" and s.leave_time > 0 for s in gone)
+    assert a.num_completion_tokens == 1, "what it had generated stays"
+    assert [it.seq for it in batch.items] == [b]
+    assert list(sched.running) == [b] and not sched.waiting
+    assert a.id not in core.manager and c.id not in core.manager
+    assert core.manager.pools[0].num_pages - core.manager.pools[0].num_free == 3
+    core.manager.check()
+    # an aborted request whose step is still running: that step's result is dropped
+    run(sched, batch)
+    batch = sched.schedule()
+    sched.abort(b.id)
+    assert sched.postprocess(batch, {b.id: 7}) == []
+    assert sched.schedule() is None
+    assert [s.id for s in sched.take_rejected()] == [b.id] and sched.is_finished()
+    assert core.manager.pools[0].num_free == core.manager.pools[0].num_pages
+
+
+def test_next_batch_info():
+    """atom/model_engine/scheduler.py:2724-2759, for steps that hold both kinds."""
+    sched, _ = make(max_num_batched_tokens=64, max_num_seqs=4)
+    assert sched.get_next_batch_info() == (False, 0, 0)
+    sched.add(seq(range(100), max_tokens=9, ignore_eos=True))
+    sched.add(seq(range(30), max_tokens=9, ignore_eos=True))
+    assert sched.get_next_batch_info() == (True, 64, 1)
+    batch = sched.schedule()
+    assert (batch.total_tokens, len(batch.items)) == (64, 1)
+    run(sched, batch)
+    assert sched.get_next_batch_info() == (True, 36, 1)      # 36 left of the first; 28 of the second are a sliver
+    batch = sched.schedule()
+    assert (batch.total_tokens, len(batch.items)) == (36, 1)
+    run(sched, batch)
+    assert sched.get_next_batch_info() == (True, 31, 2)      # one decodes, the other's 30 tokens
+    batch = sched.schedule()
+    assert (batch.total_tokens, len(batch.items)) == (31, 2)
+    run(sched, batch)
+    assert sched.get_next_batch_info() == (False, 2, 2)

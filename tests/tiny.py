@@ -27,11 +27,19 @@ TINY_C = dict(
     layer_types=["full_attention", "sliding_attention", "sliding_attention", "full_attention"],
     hidden_act="silu", torch_dtype="bfloat16")
 
+# ours: the head size of the full-size models (128) with groups of 4, a width and a vocabulary that are no
+# power of two, a tied head: the kernel variants that serving runs, at a size the plain implementation can follow
+TINY_D = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, hidden_size=264,
+    num_attention_heads=8, num_key_value_heads=2, head_dim=128, intermediate_size=328, vocab_size=1031,
+    rope_theta=1000000.0, rms_norm_eps=1e-6, max_position_embeddings=2048, tie_word_embeddings=True,
+    attention_bias=False, use_sliding_window=False, hidden_act="silu", torch_dtype="bfloat16")
+
 # the weights' spread per configuration: (linear and embedding std, norm-weight std)
-SPREAD = {"A": (0.02, 0.1), "B": (0.05, 0.2), "C": (0.04, 0.15)}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-SEEDS = {"A": 0, "B": 1, "C": 5}
-PAGE = {"A": 16, "B": 8, "C": 16}
+SPREAD = {"A": (0.02, 0.1), "B": (0.05, 0.2), "C": (0.04, 0.15), "D": (0.03, 0.1)}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+SEEDS = {"A": 0, "B": 1, "C": 5, "D": 8}
+PAGE = {"A": 16, "B": 8, "C": 16, "D": 16}
 
 
 def write_tiny(folder: str, which: str, dtype=torch.bfloat16) -> str:
