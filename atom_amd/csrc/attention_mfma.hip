@@ -44,6 +44,15 @@ struct AttnParams {
   int max_blocks, hq, hkv, page_size, window, seq_offset, parts, num_tiles;
   int page_shift;         // log2(page_size) where that is a power of two, else -1
   float scale_log2;       // softmax scale * log2(e)
+  // decode with the step before attention folded in: q is not read; the float32 QKV product is
+  const float* qkv;       // [tokens, (Hq + 2 Hkv) * D], rows q | k | v
+  const float* q_weight;  // per-head RMS norm weights [D], or null for no norm
+  const float* k_weight;
+  const float* cos_table; // [max_pos, D / 2]: the whole head is rotated
+  const float* sin_table;
+  const int* slots;       // [tokens] cache slot of each token's key and value (-1: none)
+  float eps;
+  int write_kv;           // 0: the keys and values are another layer's, already written
 };
 
 __device__ __forceinline__ s16x4 as_s16x4(bf16x4 v) { return __builtin_bit_cast(s16x4, v); }
@@ -341,8 +350,15 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
 // TOGETHER: the parts of a (request, KV head) are the waves of one block (at most 8: two waves a SIMD is what
 // the registers allow), which merges their results through LDS and writes the output itself; no second kernel
 // and no partial results in memory.  Otherwise a block is one wave and the merge kernel follows.
-template <int D, int RT, bool TOGETHER>
-__global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave) attention_decode32_kernel(AttnParams p) {
+//
+// FUSED: the kernel starts from the float32 QKV product of the step instead of from finished queries.  Every wave
+// norms and rotates its query rows itself (a lane's elements of a row and their rotation partners, half a head
+// on, are the same lane's, so this costs two exchanges for the sum of squares).  The wave whose keys end with
+// the new token (the last part) also norms and rotates that token's key, writes key and value to their page,
+// and puts them where the step's loads of that key and value have arrived, in LDS and in registers: the
+// loaded ones are whatever the page held before.  No other wave of the grid reads that key.
+template <int D, int RT, bool TOGETHER, bool FUSED>
+__global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave, (D <= 128 ? 2 : 1)) attention_decode32_kernel(AttnParams p) {
   constexpr int KCH = D / 32;      // k steps of the first product
   constexpr int DT = D / 16;       // output tiles along d
   constexpr int KP = D * 32 / 8 / kWave;   // 16-byte pieces of a step's 32 key rows per lane
@@ -372,20 +388,6 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave) attention_decode
   const int kb = vis0 + part * chunk;
   const int ke = min(ctx, kb + chunk);
 
-  bool row_ok[RT];
-  bf16x8 q32[RT][KCH];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    const int row = rt * 16 + r16;
-    row_ok[rt] = row < group;
-    const bf16_t* qr = p.q + ((size_t)tok0 * p.hq + head0 + row) * D;
-#pragma unroll
-    for (int j = 0; j < KCH; ++j) {
-      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (row_ok[rt]) v = *reinterpret_cast<const bf16x8*>(qr + 32 * j + 8 * g);
-      q32[rt][j] = v;
-    }
-  }
   f32x4 acc[RT][DT];
   float run_max[RT], run_sum[RT];
 #pragma unroll
@@ -427,12 +429,133 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave) attention_decode
 
   Step cur, nxt;
   if (kb < ke) load_step(kb, cur);
+  // (the first step's keys and values are on their way while the queries are made ready)
+  bool row_ok[RT];
+  bf16x8 q32[RT][KCH];
+  // the new token's key and value for the wave that owns them (FUSED): element i of the key at knew[i]
+  __shared__ __attribute__((aligned(16))) bf16_t knew_all[FUSED ? (TOGETHER ? 8 : 1) * 2 * D : 8];
+  bf16_t* knew = knew_all + (FUSED ? wave * 2 * D : 0);
+  bf16_t* vnew = knew + (FUSED ? D : 0);
+  const bool owns_new = FUSED && p.write_kv && kb <= pos0 && pos0 < ke;   // the same in all lanes
+  if constexpr (FUSED) {
+    static_assert(!FUSED || KCH % 2 == 0, "a lane must hold both halves of a rotation pair");
+    const size_t row_width = (size_t)(p.hq + 2 * p.hkv) * D;
+    const float* base = p.qkv + (size_t)tok0 * row_width;
+    const int pos = max(pos0, 0);
+    const float* cs = p.cos_table + (size_t)pos * (D / 2);
+    const float* sn = p.sin_table + (size_t)pos * (D / 2);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int row = rt * 16 + r16;
+      row_ok[rt] = row < group;
+      const float* qr = base + (size_t)(head0 + (row_ok[rt] ? row : 0)) * D;
+      float x[KCH][8];
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) {
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(qr + 32 * j + 8 * g);
+        const f32x4 hi = *reinterpret_cast<const f32x4*>(qr + 32 * j + 8 * g + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          x[j][e] = lo[e];
+          x[j][4 + e] = hi[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += x[j][e] * x[j][e];
+      }
+      if (p.q_weight) {
+        ss += __shfl_xor(ss, 16, kWave);
+        ss += __shfl_xor(ss, 32, kWave);
+        const float inv = rsqrtf(ss / (float)D + p.eps);
+#pragma unroll
+        for (int j = 0; j < KCH; ++j)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[j][e] = x[j][e] * inv * p.q_weight[32 * j + 8 * g + e];
+      }
+#pragma unroll
+      for (int j = 0; j < KCH / 2; ++j) {
+        bf16x8 first, second;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float c = cs[32 * j + 8 * g + e], sv = sn[32 * j + 8 * g + e];
+          const float x1 = x[j][e], x2 = x[j + KCH / 2][e];
+          first[e] = static_cast<bf16_t>(row_ok[rt] ? x1 * c - x2 * sv : 0.f);
+          second[e] = static_cast<bf16_t>(row_ok[rt] ? x2 * c + x1 * sv : 0.f);
+        }
+        q32[rt][j] = first;
+        q32[rt][j + KCH / 2] = second;
+      }
+    }
+    if (owns_new) {
+      // the new key: normed, rotated, to its page and to LDS; the new value: to its page and to LDS
+      const float* kr = base + (size_t)(p.hq + kvh) * D;
+      const float* vr = base + (size_t)(p.hq + p.hkv + kvh) * D;
+      float ss = 0.f;
+      for (int i = lane; i < D; i += kWave) ss += kr[i] * kr[i];
+      float inv = 1.f;
+      if (p.k_weight) inv = rsqrtf(wave_sum(ss) / (float)D + p.eps);
+      const int slot = p.slots[tok0];
+      const int page = slot / ps, off = slot - page * ps;
+      bf16_t* kdst = const_cast<bf16_t*>(p.k_cache) + (((size_t)page * p.hkv + kvh) * ps + off) * (size_t)D;
+      bf16_t* vdst = const_cast<bf16_t*>(p.v_cache) + ((size_t)page * p.hkv + kvh) * (size_t)D * ps + off;
+      for (int i = lane; i < D / 2; i += kWave) {
+        float x1 = kr[i], x2 = kr[i + D / 2];
+        if (p.k_weight) {
+          x1 = x1 * inv * p.k_weight[i];
+          x2 = x2 * inv * p.k_weight[i + D / 2];
+        }
+        const float c = cs[i], sv = sn[i];
+        const bf16_t y1 = static_cast<bf16_t>(x1 * c - x2 * sv), y2 = static_cast<bf16_t>(x2 * c + x1 * sv);
+        knew[i] = y1;
+        knew[i + D / 2] = y2;
+        if (slot >= 0) {
+          kdst[i] = y1;
+          kdst[i + D / 2] = y2;
+        }
+      }
+      for (int i = lane; i < D; i += kWave) {
+        const bf16_t v = static_cast<bf16_t>(vr[i]);
+        vnew[i] = v;
+        if (slot >= 0) vdst[(size_t)i * ps] = v;
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_wave_barrier();
+    }
+  } else {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int row = rt * 16 + r16;
+      row_ok[rt] = row < group;
+      const bf16_t* qr = p.q + ((size_t)tok0 * p.hq + head0 + row) * D;
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) {
+        bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (row_ok[rt]) v = *reinterpret_cast<const bf16x8*>(qr + 32 * j + 8 * g);
+        q32[rt][j] = v;
+      }
+    }
+  }
   for (int k0 = kb; k0 < ke; k0 += 32) {
     if (k0 + 32 < ke) load_step(k0 + 32, nxt);
 #pragma unroll
     for (int j = 0; j < KP; ++j) {
       const int q = kWave * j + lane;
       *reinterpret_cast<bf16x8*>(klds + (q / (D / 8)) * KLDS + (q % (D / 8)) * 16) = cur.k[j];
+    }
+    if (FUSED && owns_new && pos0 < k0 + 32) {
+      // this step's loads of the new token's key and value brought what the page held before: put the new ones there
+      const int at = pos0 - k0;                       // its place among the step's 32 keys
+      if (lane < D / 8)
+        *reinterpret_cast<bf16x8*>(klds + at * KLDS + lane * 16) = *reinterpret_cast<const bf16x8*>(knew + 8 * lane);
+      if (at >> 3 == g) {
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+          const bf16_t v = vnew[16 * t + r16];
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (e == (at & 7)) cur.v[t][e] = v;
+        }
+      }
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0); the block is one wave
     __builtin_amdgcn_wave_barrier();
@@ -628,7 +751,7 @@ static int page_shift_of(int page_size) {
   return shift;
 }
 
-template <int D>
+template <int D, bool FUSED>
 static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
   const int group = p.hq / p.hkv;
   dim3 grid(p.parts, p.hkv, seqs), block(kWave);
@@ -641,28 +764,32 @@ static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
         // the parts of a (request, KV head) as the waves of one block, which merges them itself
         // (up to 16 heads a KV head: their results fit where a wave kept its key rows)
         static bool allowed = false;
-        if (!allowed && hipFuncSetAttribute((const void*)attention_decode32_kernel<D, 1, true>,
+        if (!allowed && hipFuncSetAttribute((const void*)attention_decode32_kernel<D, 1, true, FUSED>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize, 8 * area) != hipSuccess)
           return ATOM_LAUNCH_FAILED;
         allowed = true;
-        hipLaunchKernelGGL((attention_decode32_kernel<D, 1, true>), dim3(1, p.hkv, seqs), dim3(p.parts * kWave),
+        hipLaunchKernelGGL((attention_decode32_kernel<D, 1, true, FUSED>), dim3(1, p.hkv, seqs), dim3(p.parts * kWave),
                            area * p.parts, stream, p);
         return launch_status();
       }
-      if (group <= 16) hipLaunchKernelGGL((attention_decode32_kernel<D, 1, false>), grid, block, area, stream, p);
-      else hipLaunchKernelGGL((attention_decode32_kernel<D, 2, false>), grid, block, area, stream, p);
-    } else {
-      if (group <= 16) hipLaunchKernelGGL((attention_mfma_kernel<D, 1, true>), grid, block, 0, stream, p);
-      else hipLaunchKernelGGL((attention_mfma_kernel<D, 2, true>), grid, block, 0, stream, p);
+      if (group <= 16) hipLaunchKernelGGL((attention_decode32_kernel<D, 1, false, FUSED>), grid, block, area, stream, p);
+      else hipLaunchKernelGGL((attention_decode32_kernel<D, 2, false, FUSED>), grid, block, area, stream, p);
+      if (p.parts > 1)
+        hipLaunchKernelGGL(attention_merge_kernel, dim3(p.hq, seqs), dim3(kMergeGroups * kWave), 0, stream, p.ws_o,
+                           p.ws_ml, p.out, p.cu_q, p.seq_offset, p.hq, D, p.parts);
+      return launch_status();
     }
+  }
+  if constexpr (FUSED) {
+    return ATOM_UNSUPPORTED;
   } else {
     if (group <= 16) hipLaunchKernelGGL((attention_mfma_kernel<D, 1, true>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((attention_mfma_kernel<D, 2, true>), grid, block, 0, stream, p);
+    if (p.parts > 1)
+      hipLaunchKernelGGL(attention_merge_kernel, dim3(p.hq, seqs), dim3(kMergeGroups * kWave), 0, stream, p.ws_o,
+                         p.ws_ml, p.out, p.cu_q, p.seq_offset, p.hq, D, p.parts);
+    return launch_status();
   }
-  if (p.parts > 1)
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(p.hq, seqs), dim3(kMergeGroups * kWave), 0, stream, p.ws_o,
-                       p.ws_ml, p.out, p.cu_q, p.seq_offset, p.hq, D, p.parts);
-  return launch_status();
 }
 
 // ------------------------------------------------------------------ prefill with shared key tiles
@@ -1020,10 +1147,52 @@ ATOM_EXPORT int atom_attention_decode(const void* q, const void* k_cache, const 
   p.ws_o = ws_o; p.ws_ml = ws_ml; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
   p.window = window; p.seq_offset = seq_offset; p.parts = parts; p.scale_log2 = scale * 1.4426950408889634f;
   p.page_shift = page_shift_of(page_size);
-#define CALL(DD) return launch_decode<DD>(p, seqs, stream)
+#define CALL(DD) return launch_decode<DD, false>(p, seqs, stream)
   ATOM_FOR_HEAD_DIM(d, CALL)
 #undef CALL
   return ATOM_OK;
+}
+
+// 1 if atom_attention_decode_fused takes this head size, page size and group: the head sizes whose rotation
+// pairs lie in one lane, pages of a multiple of 8 keys.
+ATOM_EXPORT int atom_attention_decode_fused_supports(int d, int page_size, int group) {
+  return (d == 64 || d == 128 || d == 256) && page_size > 0 && page_size % 8 == 0 && group >= 1 && group <= 32;
+}
+
+// Decode attention that starts from the step's float32 QKV product [tokens, (Hq + 2 Hkv) * D]: per-head RMS norm
+// of q and k (weights may be null), rotation of the whole head by the tables at each request's last position,
+// the new key and value written at slots[token] (write_kv), attention over the pages.  Otherwise as
+// atom_attention_decode.
+ATOM_EXPORT int atom_attention_decode_fused(const float* qkv, const float* q_weight, const float* k_weight,
+                                            const float* cos_table, const float* sin_table, const int* slots,
+                                            float eps, int write_kv, void* k_cache, void* v_cache, void* out,
+                                            const int* cu_q, const int* ctx_lens, const int* block_tables,
+                                            int max_blocks, int seq_offset, int seqs, int hq, int hkv, int d,
+                                            int page_size, float scale, int window, int parts, float* ws_o,
+                                            float* ws_ml, hipStream_t stream) {
+  if (int st = check_common(hq, hkv, d, page_size, max_blocks)) return st;
+  if (!atom_attention_decode_fused_supports(d, page_size, hq / hkv)) return ATOM_UNSUPPORTED;
+  if (seqs < 0 || parts < 1 || seq_offset < 0 || !qkv || !cos_table || !sin_table) return ATOM_BAD_SHAPE;
+  if (write_kv && (!slots || !k_cache || !v_cache)) return ATOM_BAD_SHAPE;
+  if (parts > kWave) return ATOM_TOO_LARGE;
+  if (parts > 1 && (!ws_o || !ws_ml)) return ATOM_BAD_SHAPE;
+  if (seqs > 65535 || hkv > 65535) return ATOM_TOO_LARGE;
+  if (((uintptr_t)qkv) & 15) return ATOM_BAD_SHAPE;
+  if (seqs == 0) return ATOM_OK;
+  AttnParams p{};
+  p.q = nullptr; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache;
+  p.out = (bf16_t*)out; p.cu_q = cu_q; p.ctx_lens = ctx_lens; p.block_tables = block_tables; p.tiles = nullptr;
+  p.ws_o = ws_o; p.ws_ml = ws_ml; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
+  p.window = window; p.seq_offset = seq_offset; p.parts = parts; p.scale_log2 = scale * 1.4426950408889634f;
+  p.page_shift = page_shift_of(page_size);
+  p.qkv = qkv; p.q_weight = q_weight; p.k_weight = k_weight; p.cos_table = cos_table; p.sin_table = sin_table;
+  p.slots = slots; p.eps = eps; p.write_kv = write_kv;
+  switch (d) {
+    case 64: return launch_decode<64, true>(p, seqs, stream);
+    case 128: return launch_decode<128, true>(p, seqs, stream);
+    case 256: return launch_decode<256, true>(p, seqs, stream);
+    default: return ATOM_UNSUPPORTED;
+  }
 }
 
 // Prefill: `tiles` lists (request, first row) for every tile of `rows_per_tile` query tokens: 16 or 32 for

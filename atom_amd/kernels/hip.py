@@ -90,6 +90,41 @@ class DeferredSum:
         return self.partial.shape[1] * self.partial.shape[2]
 
 
+class PendingNorm:
+    """An RMS norm that has not been applied yet: float32 rows ``r`` [*, width]; ``xg`` = bfloat16(r * weight),
+    the same rows times the norm's weight; ``ss`` [*, parts], partial sums of squares of the rows of ``r`` (all
+    three left by the product that wrote ``r``); eps; and optionally which rows are meant (``rows``, int32).  The
+    few-rows product takes ``xg`` as its input and multiplies its float32 sums by the rows' 1 / rms
+    (``HipKernels.linear`` / ``linear_silu``); ``HipKernels.materialize`` runs the norm kernel on ``r``."""
+
+    def __init__(self, r, xg, ss, weight, eps: float, rows, dtype: torch.dtype):
+        self.r, self.xg, self.ss, self.weight, self.eps, self.rows, self.dtype = r, xg, ss, weight, float(eps), rows, dtype
+
+    @property
+    def shape(self):
+        return torch.Size((self.rows.numel() if self.rows is not None else self.r.shape[0], self.r.shape[1]))
+
+    @property
+    def device(self):
+        return self.r.device
+
+
+class PendingProduct:
+    """``x @ weight.T (+ bias)`` of few rows that has not been launched: what follows decides its epilogue (a norm
+    with the residual stream adds the sum in place; anything else takes the plain product)."""
+
+    def __init__(self, x, weight, bias, dtype: torch.dtype):
+        self.x, self.weight, self.bias, self.dtype = x, weight, bias, dtype
+
+    @property
+    def shape(self):
+        return torch.Size((self.x.shape[0], self.weight.shape[0]))
+
+    @property
+    def device(self):
+        return self.weight.device
+
+
 def _ptr(t: torch.Tensor | None):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else None
 
@@ -115,15 +150,21 @@ class HipKernels:
                    "atom_gemm_skinny", "atom_gemm_skinny_splits", "atom_gemm_skinny_supports", "atom_splitk_reduce",
                    "atom_paged_attention_generic", "atom_gemm_f32", "atom_sample", "atom_exponential_noise",
                    "atom_attention_mfma_supports", "atom_attention_decode", "atom_attention_prefill",
-                   "atom_attention_prefill_tile_rows"):
+                   "atom_attention_prefill_tile_rows", "atom_attention_decode_fused",
+                   "atom_attention_decode_fused_supports", "atom_gemm_rows", "atom_gemm_rows_parts",
+                   "atom_gemm_rows_supports"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
         # up to 128 for the narrow products that atom_gemm_skinny_supports names; the BLAS library takes the rest.
         self.use_skinny_gemm = True
         self.skinny_max_rows = 128
+        # up to 8 bfloat16 rows: the product with the norm before it and the residual sum after it folded in
+        self.use_rows_gemm = True
+        self.rows_waves = 0     # 4 or 8 forces the waves a block of that kernel (0: its own choice)
         self.use_mfma_attention = True
         self.use_tiled_prefill = True
+        self.use_fused_decode = True    # decode-only steps of few rows: norm, rotation and cache write inside attention
         self._ws: dict[str, torch.Tensor] = {}
         self._zeroed: dict[str, torch.Tensor] = {}   # workspaces that every kernel leaves all zero
         self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
@@ -232,7 +273,13 @@ class HipKernels:
         return None, 0, ctypes.c_long(0), None
 
     def materialize(self, x):
-        """A tensor from what may still be a sum of slices."""
+        """A tensor from what may still be a sum of slices, a product not launched yet or a norm not applied yet."""
+        if isinstance(x, PendingProduct):
+            return self._rows_product(x.x, x.weight, x.bias, x.dtype)
+        if isinstance(x, PendingNorm):
+            out = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
+            # the float32 rows as a sum of one slice: the norm kernel reads float32 and writes the step's type
+            return self.rmsnorm(DeferredSum(x.r.unsqueeze(0), None, x.dtype), x.weight, x.eps, out, rows=x.rows)
         if not isinstance(x, DeferredSum):
             return x
         rows, width = x.shape
@@ -241,6 +288,56 @@ class HipKernels:
             _ptr(x.partial), _ptr(x.bias), _ptr(y), rows, width, x.splits, int(x.dtype == torch.float32),
             self._stream()))
         return y
+
+    # ---- the few-rows product with the norm before it and the residual sum after it folded in
+
+    def _rows_takes(self, x, weight) -> bool:
+        m, k = x.shape
+        return bool(self.use_rows_gemm and 1 <= m <= 8 and weight.dtype == torch.bfloat16
+                    and (isinstance(x, PendingNorm) or x.dtype == torch.bfloat16)
+                    and self.lib.atom_gemm_rows_supports(m, weight.shape[0], k))
+
+    def _rows_launch(self, x, weight, bias, mode: int, y=None, res=None, ss_out=None, xg_out=None, g_next=None,
+                     out_f32: bool = False):
+        m, k = x.shape
+        n = weight.shape[0] // 2 if mode == 1 else weight.shape[0]
+        self._check("linear weight", weight, torch.bfloat16, (weight.shape[0], k))
+        if bias is not None:
+            self._check("linear bias", bias, torch.float32, (weight.shape[0],))
+        if isinstance(x, PendingNorm):
+            self._check("norm input", x.xg, torch.bfloat16, (None, k))
+            self._check("sums of squares", x.ss, torch.float32, (x.xg.shape[0], None))
+            if x.rows is not None:
+                self._check("norm row choice", x.rows, torch.int32, (m,))
+            head = (_ptr(x.xg), _ptr(x.rows), _ptr(x.ss), x.ss.shape[1], ctypes.c_float(x.eps))
+        else:
+            self._check("linear input", x, torch.bfloat16, (m, k))
+            head = (_ptr(x), None, None, 0, ctypes.c_float(0.0))
+        self._done("gemm_rows", self.lib.atom_gemm_rows(
+            *head, _ptr(weight), _ptr(bias), _ptr(y), _ptr(res), _ptr(ss_out), _ptr(xg_out), _ptr(g_next), m, n, k,
+            mode, int(out_f32), int(self.rows_waves), self._stream()))
+
+    def _rows_product(self, x, weight, bias, out_dtype):
+        y = torch.empty((x.shape[0], weight.shape[0]), dtype=out_dtype, device=weight.device)
+        self._rows_launch(x, weight, bias, 0, y=y, out_f32=out_dtype == torch.float32)
+        return y
+
+    def pending_norm(self, x, residual, weight, eps: float, rows=None):
+        """``residual += x`` where x is a product that has not been launched (it is launched now, the sum formed
+        in place where the product leaves the matrix cores), and the norm of the sum left pending for the product
+        that follows.  None if ``x`` is anything else: the caller then takes ``rmsnorm``."""
+        if not isinstance(x, PendingProduct) or residual is None:
+            return None
+        m, n = x.shape
+        self._check("residual", residual, torch.float32, (m, n))
+        self._check("norm weight", weight, torch.float32, (n,))
+        inner = x.x
+        if isinstance(inner, PendingNorm) and inner.r.data_ptr() == residual.data_ptr():
+            inner = self.materialize(inner)   # the product may not read the rows it adds to
+        ss = torch.empty((m, self.lib.atom_gemm_rows_parts(n)), dtype=torch.float32, device=residual.device)
+        xg = torch.empty((m, n), dtype=torch.bfloat16, device=residual.device)
+        self._rows_launch(inner, x.weight, x.bias, 2, res=residual, ss_out=ss, xg_out=xg, g_next=weight)
+        return PendingNorm(residual, xg, ss, weight, eps, rows, x.dtype)
 
     # ------------------------------------------------------------------ kernels
 
@@ -270,6 +367,8 @@ class HipKernels:
         """mode 'plain': out = norm(x); 'init': residual = x, out = norm(x);
         'add': residual += x, out = norm(residual).  With ``rows`` only those source
         rows are normed (into out[0..len(rows))) and the residual is not written."""
+        if isinstance(x, (PendingProduct, PendingNorm)):
+            x = self.materialize(x)
         width = x.shape[-1]
         code = {"plain": 0, "init": 1, "add": 2}[mode]
         deferred = isinstance(x, DeferredSum)
@@ -304,6 +403,10 @@ class HipKernels:
     def qk_norm_rope_kv_write(self, qkv, q_out, k_cache, v_cache, q_weight, k_weight, cos, sin, positions,
                               slots, num_heads: int, num_kv_heads: int, head_dim: int, rotary_dim: int,
                               page_size: int, eps: float, write_kv: bool = True):
+        if isinstance(qkv, PendingProduct):
+            # the float32 product as a sum of one slice: the kernel reads it with the precision it reads slices
+            full = self._rows_product(qkv.x, qkv.weight, qkv.bias, torch.float32)
+            qkv = DeferredSum(full.unsqueeze(0), None, qkv.dtype)
         tokens = qkv.shape[0]
         dt = qkv.dtype
         deferred = isinstance(qkv, DeferredSum)
@@ -370,6 +473,55 @@ class HipKernels:
                 int(window or 0), parts, _ptr(ws_o), _ptr(ws_ml), self._stream()))
         return out
 
+    def fused_decode_attention(self, qkv, k_cache, v_cache, out, meta: AttentionMeta, scale: float, window, q_weight,
+                               k_weight, cos, sin, slots, num_heads: int, num_kv_heads: int, head_dim: int,
+                               rotary_dim: int, eps: float, write_kv: bool = True, parts: int | None = None):
+        """For a step in which every request brings one token: per-head norm of q and k, rotation, the write of the
+        new keys and values and attention over the pages in one kernel (and the merge of the key ranges), starting
+        from the QKV product, which has to be one that has not been launched yet (a few-rows ``PendingProduct``; it is
+        launched here with float32 output).  Returns ``out``, or None when this case is not taken: the caller then
+        runs ``qk_norm_rope_kv_write`` and ``paged_attention``."""
+        page_size = meta.page_size
+        if (not self.use_fused_decode or not isinstance(qkv, PendingProduct) or meta.num_prefill or out.dtype != torch.bfloat16
+                or rotary_dim != head_dim or cos is None
+                or not self.lib.atom_attention_decode_fused_supports(head_dim, page_size, num_heads // num_kv_heads)):
+            return None
+        tokens = qkv.shape[0]
+        if meta.num_seqs != tokens or tuple(qkv.shape) != (tokens, (num_heads + 2 * num_kv_heads) * head_dim):
+            return None
+        self._check("key pages", k_cache, torch.bfloat16, (None, num_kv_heads, page_size, head_dim))
+        self._check("value pages", v_cache, torch.bfloat16, (k_cache.shape[0], num_kv_heads, head_dim, page_size))
+        self._check("attention out", out, torch.bfloat16, (tokens, num_heads, head_dim))
+        self._check("cu_seqlens_q", meta.cu_seqlens_q, torch.int32, (tokens + 1,))
+        self._check("context_lens", meta.context_lens, torch.int32, (tokens,))
+        self._check("block tables", meta.block_tables, torch.int32, (tokens, None))
+        self._check("cos table", cos, torch.float32, (None, head_dim // 2))
+        self._check("sin table", sin, torch.float32, tuple(cos.shape))
+        if meta.max_context_len > cos.shape[0]:
+            raise KernelError("attention: a position lies beyond the rotation tables")
+        if meta.max_context_len > meta.block_tables.shape[1] * page_size:
+            raise KernelError("attention: a context is longer than its block table can name")
+        for name, w in (("q norm weight", q_weight), ("k norm weight", k_weight)):
+            if w is not None:
+                self._check(name, w, torch.float32, (head_dim,))
+        if write_kv:
+            self._check("slot mapping", slots, torch.int32, (tokens,))
+        full = self._rows_product(qkv.x, qkv.weight, qkv.bias, torch.float32)
+        if parts is None:
+            visible = min(meta.max_context_len, window) if window else meta.max_context_len
+            parts = self.decode_parts(tokens, num_kv_heads, visible)
+        ws_o = ws_ml = None
+        if parts > 1:
+            ws_o = self.workspace("attn_o", tokens * num_heads * parts * head_dim)
+            ws_ml = self.workspace("attn_ml", tokens * num_heads * parts * 2)
+        bt = meta.block_tables
+        self._done("attention_decode_fused", self.lib.atom_attention_decode_fused(
+            _ptr(full), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin), _ptr(slots) if write_kv else None,
+            ctypes.c_float(eps), int(bool(write_kv)), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.cu_seqlens_q),
+            _ptr(meta.context_lens), _ptr(bt), bt.shape[1], 0, tokens, num_heads, num_kv_heads, head_dim, page_size,
+            ctypes.c_float(scale), int(window or 0), parts, _ptr(ws_o), _ptr(ws_ml), self._stream()))
+        return out
+
     def paged_attention(self, q, k_cache, v_cache, out, meta: AttentionMeta, scale: float,
                         window: int | None = None, parts: int | None = None):
         tokens, hq, d = q.shape
@@ -409,8 +561,15 @@ class HipKernels:
         does for its matrix products; anything with a float32 operand runs this library's float32
         kernel (plain FMA, no reduced-precision mode).  With ``defer`` the result may come back as a
         ``DeferredSum`` for a kernel that adds the slices while it reads them."""
+        if isinstance(x, (DeferredSum, PendingProduct)):
+            x = self.materialize(x)
         m, k = x.shape
         n = weight.shape[0]
+        if m and self._rows_takes(x, weight):
+            if defer:
+                return PendingProduct(x, weight, bias, out_dtype or x.dtype)
+            return self._rows_product(x, weight, bias, out_dtype or x.dtype)
+        x = self.materialize(x)
         self._check("linear input", x, (torch.float32, torch.bfloat16))
         self._check("linear weight", weight, (torch.float32, torch.bfloat16), (n, k))
         out_dtype = out_dtype or x.dtype
@@ -452,6 +611,11 @@ class HipKernels:
         if two % 2:
             raise KernelError("linear_silu: the weight must hold as many gate rows as up rows")
         inter = two // 2
+        if m and self._rows_takes(x, weight):
+            act = torch.empty((m, inter), dtype=x.dtype, device=weight.device)
+            self._rows_launch(x, weight, bias, 1, y=act)
+            return act
+        x = self.materialize(x)
         if m and self._skinny(x, weight):
             self._check("linear input", x, torch.bfloat16)
             self._check("linear weight", weight, torch.bfloat16, (two, k))

@@ -19,6 +19,7 @@ from .base import MIXERS, POSITION_ENCODINGS, KVCacheNeed, Mixer, ParamSpec, Par
 
 class GroupedQueryAttention(Mixer):
     graph_safe = True
+    accepts_deferred = True   # the input goes to the QKV product as it is
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool = False, out_bias: bool = False, qk_norm: bool = False, norm_eps: float = 1e-6,
@@ -115,16 +116,25 @@ class GroupedQueryAttention(Mixer):
         ops = ctx.ops
         tokens = x.shape[0]
         qkv = ops.linear(x, self.params["qkv.weight"], self.p("qkv.bias"), defer=True)
-        q = torch.empty((tokens, self.num_heads, self.head_dim), dtype=x.dtype, device=x.device)
         meta = self._meta(ctx, cache.group)
         rope = self.rope
-        ops.qk_norm_rope_kv_write(
-            qkv, q, cache.k_cache, cache.v_cache, self.p("q_norm.weight"), self.p("k_norm.weight"),
-            rope.cos if rope else None, rope.sin if rope else None, ctx.positions,
-            ctx.slot_mappings[cache.group], self.num_heads, self.num_kv_heads, self.head_dim,
-            rope.rotary_dim if rope else 0, meta.page_size, self.norm_eps, write_kv=cache.writes)
-        out = torch.empty_like(q)
-        ops.paged_attention(q, cache.k_cache, cache.v_cache, out, meta, self.scale, self.window)
+        out = torch.empty((tokens, self.num_heads, self.head_dim), dtype=x.dtype, device=x.device)
+        fused = getattr(ops, "fused_decode_attention", None)
+        done = None
+        if fused is not None and rope is not None:
+            # a decode step of few requests: one kernel from the QKV product to the attention output
+            done = fused(qkv, cache.k_cache, cache.v_cache, out, meta, self.scale, self.window,
+                         self.p("q_norm.weight"), self.p("k_norm.weight"), rope.cos, rope.sin,
+                         ctx.slot_mappings[cache.group], self.num_heads, self.num_kv_heads, self.head_dim,
+                         rope.rotary_dim, self.norm_eps, write_kv=cache.writes)
+        if done is None:
+            q = torch.empty((tokens, self.num_heads, self.head_dim), dtype=x.dtype, device=x.device)
+            ops.qk_norm_rope_kv_write(
+                qkv, q, cache.k_cache, cache.v_cache, self.p("q_norm.weight"), self.p("k_norm.weight"),
+                rope.cos if rope else None, rope.sin if rope else None, ctx.positions,
+                ctx.slot_mappings[cache.group], self.num_heads, self.num_kv_heads, self.head_dim,
+                rope.rotary_dim if rope else 0, meta.page_size, self.norm_eps, write_kv=cache.writes)
+            ops.paged_attention(q, cache.k_cache, cache.v_cache, out, meta, self.scale, self.window)
         return ops.linear(out.view(tokens, self.num_heads * self.head_dim), self.params["o.weight"], self.p("o.bias"),
                           defer=True)
 

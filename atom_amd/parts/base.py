@@ -140,6 +140,10 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    #: True when ``forward`` hands its input to ``ctx.ops.linear`` / ``linear_silu`` as it is and reads nothing of
+    #: it but ``shape``, ``dtype`` and ``device``: the norm before the mixer may then be left to that product
+    #: (the input is a ``PendingNorm``).  Other mixers always get a tensor.
+    accepts_deferred = False
     #: True when ``forward`` launches the same kernels whatever the batch holds and reads the batch
     #: only through device arrays of ``ctx``: a decode step of such mixers may be replayed as a HIP graph
     graph_safe = False
@@ -169,6 +173,9 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    #: as ``Mixer.accepts_deferred``
+    accepts_deferred = False
+
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 

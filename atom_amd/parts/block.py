@@ -30,10 +30,14 @@ class PreNormBlock(Block):
         if not self.mixer_norm.accepts_deferred:
             hidden = ctx.ops.materialize(hidden)
         hidden, residual = self.mixer_norm.forward_residual(ctx, hidden, residual)
+        if not self._mixer.accepts_deferred:
+            hidden = ctx.ops.materialize(hidden)
         hidden = self._mixer.forward(ctx, hidden, cache)
         if not self.ffn_norm.accepts_deferred:
             hidden = ctx.ops.materialize(hidden)
         hidden, residual = self.ffn_norm.forward_residual(ctx, hidden, residual)
+        if not self.ffn.accepts_deferred:
+            hidden = ctx.ops.materialize(hidden)
         hidden = self.ffn.forward(ctx, hidden)
         return hidden, residual
 

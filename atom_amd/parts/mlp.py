@@ -8,6 +8,8 @@ from .base import FEED_FORWARDS, FeedForward, ParamSpec
 
 
 class GatedMLP(FeedForward):
+    accepts_deferred = True   # the input goes to the gate/up product as it is
+
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", bias: bool = False,
                  prefix: str = "", names: dict[str, str] | None = None):
         super().__init__(prefix)

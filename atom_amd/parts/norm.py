@@ -24,6 +24,13 @@ class RMSNorm(Norm):
         return ctx.ops.rmsnorm(x, self.params["weight"], self.eps, out)
 
     def forward_residual(self, ctx, x, residual):
+        pending = getattr(ctx.ops, "pending_norm", None)
+        if pending is not None and residual is not None:
+            # a product that has not been launched takes the residual sum as its epilogue and leaves the norm
+            # to the product that follows
+            lazy = pending(x, residual, self.params["weight"], self.eps)
+            if lazy is not None:
+                return lazy, residual
         out = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
         if residual is None:
             residual = torch.empty(tuple(x.shape), dtype=torch.float32, device=x.device)
@@ -33,6 +40,11 @@ class RMSNorm(Norm):
         return out, residual
 
     def forward_rows(self, ctx, x, residual, rows):
+        pending = getattr(ctx.ops, "pending_norm", None)
+        if pending is not None and residual is not None:
+            lazy = pending(x, residual, self.params["weight"], self.eps, rows)
+            if lazy is not None:
+                return lazy
         out = torch.empty((rows.numel(), self.size), dtype=x.dtype, device=x.device)
         mode = "add" if residual is not None else "plain"
         return ctx.ops.rmsnorm(x, self.params["weight"], self.eps, out, residual=residual, mode=mode, rows=rows)

@@ -1,7 +1,7 @@
 #!/usr/bin/python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape 8b|4b|32b]
 
 The default run has the layer sizes of Qwen3-8B (36 layers, hidden 4096, 32/8 heads of
 128, intermediate 12288, vocabulary 151936) with seeded random bfloat16 weights, 8
@@ -9,6 +9,14 @@ sequences of 2,048 random prompt tokens each, and times K decode steps through t
 engine's own step loop (scheduler, step function, sampler).  ``value`` is decoded tokens
 a second.  It also times one 2,048-token prefill and decoding at batch 1 and 64, and
 prints one JSON line.  More than one GPU is not built: ``--gpus N>1`` says so and exits 2.
+
+``--shape 4b`` runs the Qwen3-4B shape (hidden 2560 under 32 heads of 128, tied head) on its
+workload: 32 requests with prompts of 64 to 3,072 tokens through the scheduler, prompt portions
+of 512 tokens beside the running requests' decode tokens, 128 output tokens each.
+``--shape 32b`` runs the Qwen3-32B shape (64 layers, 65 GB of weights) on its workload:
+8,192-token prompts prefilled in portions, then 16 requests decoding 256 tokens, with the
+cache pool sized from the memory that is left (``num_kvcache_blocks=-1``).  Each prints one
+JSON line of the same form.
 """
 
 from __future__ import annotations
@@ -26,6 +34,11 @@ QWEN3_8B = dict(
     num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936,
     rope_theta=1000000.0, rms_norm_eps=1e-6, max_position_embeddings=40960, tie_word_embeddings=False,
     attention_bias=False, use_sliding_window=False, hidden_act="silu", torch_dtype="bfloat16")
+
+
+QWEN3_4B = dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, tie_word_embeddings=True)
+QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
+SHAPES = {"8b": ("Qwen3-8B", QWEN3_8B, 2), "4b": ("Qwen3-4B", QWEN3_4B, 3), "32b": ("Qwen3-32B", QWEN3_32B, 4)}
 
 
 def weight_bytes(c: dict, layers: int, elem: int = 2) -> int:
@@ -51,11 +64,152 @@ def prefill_flops(c: dict, layers: int, tokens: int) -> float:
     return gemm + attn + head
 
 
+def flat_config(name: str, raw: dict, layers: int, **more) -> dict:
+    """Every size of the run, flat (at most 20 keys)."""
+    cfg = {"model": f"{name} shape, random weights", "parallelism": "single GPU", "layers": layers,
+           "layers_of_model": raw["num_hidden_layers"], "hidden_size": raw["hidden_size"],
+           "num_attention_heads": raw["num_attention_heads"], "num_key_value_heads": raw["num_key_value_heads"],
+           "head_dim": raw["head_dim"], "intermediate_size": raw["intermediate_size"], "vocab_size": raw["vocab_size"],
+           "tied_head": raw["tie_word_embeddings"], "kv_block_size": 16}
+    cfg.update(more)
+    assert len(cfg) <= 20
+    return cfg
+
+
+class ByteCounter:
+    """Wraps the step function: adds up what every step has to read at least, the weights once and the
+    cache of the requests in it, and the steps' matrix-product flops."""
+
+    def __init__(self, core, raw, layers):
+        self.core, self.inner = core, core.step
+        self.weights = weight_bytes(raw, layers)
+        self.kv = kv_bytes_per_token(raw, layers)
+        h, d = raw["hidden_size"], raw["head_dim"]
+        hq, hkv, inter = raw["num_attention_heads"], raw["num_key_value_heads"], raw["intermediate_size"]
+        self.flops_per_token = 2.0 * layers * (h * (hq + 2 * hkv) * d + hq * d * h + 3 * inter * h)
+        self.head_flops = 2.0 * raw["vocab_size"] * h
+        self.attn_flops_per_pair = 4.0 * layers * hq * d
+        self.reset()
+        core.step = self.step
+
+    def reset(self):
+        self.bytes = self.flops = 0.0
+        self.steps = self.tokens = 0
+
+    def step(self, entries):
+        for e in entries:
+            before = self.core.num_cached(e.req_id)
+            n = len(e.tokens)
+            self.bytes += (before + n) * self.kv
+            self.flops += n * self.flops_per_token + len(e.want) * self.head_flops
+            self.flops += self.attn_flops_per_pair * (n * before + n * (n + 1) / 2)
+            self.tokens += n
+        self.bytes += self.weights
+        self.steps += 1
+        return self.inner(entries)
+
+
+def run_mixed(llm, args, name, raw, layers, gen, requests: int) -> dict:
+    """Continuous batching under load: every step holds the running requests' decode tokens and, under a
+    budget of 512 + N tokens, the next portion of a waiting prompt."""
+    import torch
+    from atom_amd import SamplingParams
+
+    vocab = raw["vocab_size"]
+    llm.scheduler.max_num_batched_tokens = 512 + requests
+    sp = SamplingParams(temperature=0.0, max_tokens=128, ignore_eos=True)
+    warm = [torch.randint(0, vocab, (n,), generator=gen).tolist() for n in (700, 90)]
+    llm.generate(warm, SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))   # untimed: first-use work
+    lens = torch.randint(64, 3073, (requests,), generator=gen).tolist()
+    prompts = [torch.randint(0, vocab, (n,), generator=gen).tolist() for n in lens]
+    counter = ByteCounter(llm.core, raw, layers)
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    outs = llm.generate(prompts, sp)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t
+    assert all(o["num_tokens_output"] == 128 for o in outs)
+    out_tokens = 128 * requests
+    return {
+        "metric": f"output tok/s of {requests} mixed requests, prompt portions of 512 beside decodes ({name}, bf16)",
+        "value": round(out_tokens / elapsed, 1), "unit": "tokens/s", "n_gpus": 1, "steps": counter.steps, "warmup": 0,
+        "ms_per_step": round(elapsed / counter.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic: seeded uniform random token ids and prompt lengths, seeded random N(0, 0.02) weights",
+        "config": flat_config(name, raw, layers, global_batch=requests, seq_len=3072, prompt_tokens=sum(lens),
+                              output_tokens=out_tokens, portion=512, max_model_len=llm.config.max_model_len,
+                              hip_graphs=not args.enforce_eager),
+        "roofline": {"bound": "hbm", "achieved": round(counter.bytes / elapsed / 1e9, 1), "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": round(counter.bytes / elapsed / HBM_PEAK, 4)},
+        "mfma_frac": round(counter.flops / elapsed / MFMA_PEAK["bf16"], 4),
+        "total_tok_s": round((sum(lens) + out_tokens) / elapsed, 1), "seconds": round(elapsed, 3),
+        "preemptions": llm.scheduler.total_preemptions,
+        "mean_ttft_ms": round(1e3 * sum(o["ttft"] for o in outs) / len(outs), 1),
+        "mean_tpot_ms": round(1e3 * sum(o["tpot"] for o in outs) / len(outs), 2),
+    }
+
+
+def run_long(llm, args, name, raw, layers, gen, batch: int = 16, prompt_len: int = 8192, out_tokens: int = 256) -> dict:
+    """Long prompts prefilled in portions of the token budget, then the whole batch decodes."""
+    import torch
+    from atom_amd import SamplingParams
+
+    vocab = raw["vocab_size"]
+    llm.generate([torch.randint(0, vocab, (600,), generator=gen).tolist()],
+                 SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))            # untimed: first-use work
+    sp = SamplingParams(temperature=0.0, max_tokens=out_tokens, ignore_eos=True)
+    for _ in range(batch):
+        llm.add_request(torch.randint(0, vocab, (prompt_len,), generator=gen).tolist(), sp)
+    counter = ByteCounter(llm.core, raw, layers)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while any(s.num_completion_tokens == 0 for s in llm.seqs.values()):
+        llm.step()
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    prefill_steps, prefill_flops = counter.steps, counter.flops
+    print(f"[bench] {batch} prompts of {prompt_len} tokens prefilled in {t_prefill:.2f} s, {prefill_steps} steps",
+          file=sys.stderr, flush=True)
+    for _ in range(args.warmup):
+        llm.step()
+    torch.cuda.synchronize()
+    assert len(llm.scheduler.running) == batch and not llm.scheduler.waiting
+    steps = min(args.steps, out_tokens - args.warmup - batch - 8)
+    counter.reset()
+    t = time.perf_counter()
+    for _ in range(steps):
+        llm.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t
+    assert len(llm.scheduler.running) == batch, "a request finished inside the timed steps"
+    step_bytes = counter.bytes / counter.steps
+    while not llm.is_finished():
+        llm.step()
+    llm.seqs.clear()
+    pool = llm.core.plan.groups[0]
+    return {
+        "metric": f"decode tok/s at batch {batch} after {prompt_len}-token prompts ({name}, bf16)",
+        "value": round(batch * steps / elapsed, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic: seeded uniform random token ids, seeded random N(0, 0.02) weights",
+        "config": flat_config(name, raw, layers, global_batch=batch, seq_len=prompt_len, max_model_len=llm.config.max_model_len,
+                              portion=llm.config.max_num_batched_tokens, cache_pages=pool.num_pages,
+                              cache_gb=round(llm.core.plan.total_bytes() / 1e9, 1), hip_graphs=not args.enforce_eager),
+        "prefill": {"value": round(batch * prompt_len / t_prefill, 1), "tokens": batch * prompt_len,
+                    "ms": round(t_prefill * 1e3, 1), "frac": round(prefill_flops / t_prefill / MFMA_PEAK["bf16"], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(step_bytes * steps / elapsed / 1e9, 1), "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": round(step_bytes * steps / elapsed / HBM_PEAK, 4)},
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
+                    help="8b: decode at batch 8 (and 1, 64) and a 2,048-token prefill; 4b: 32 mixed requests; "
+                         "32b: 8,192-token prompts in portions, then decode at batch 16 with the cache sized from memory")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
     ap.add_argument("--max-model-len", type=int, default=None,
@@ -64,8 +218,7 @@ def main() -> int:
     ap.add_argument("--points", type=str, default="1,64", help="other decode batch sizes to time")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
-                    help="instead: N requests with prompts of 64..3072 tokens through the scheduler, prompt portions of "
-                         "512 tokens beside running decodes, 128 output tokens each; prints its own line")
+                    help="the mixed workload with N requests on the chosen shape (what --shape 4b runs with 32)")
     ap.add_argument("--temperature", type=float, default=0.0, help="of the decode steps' sampling (0: greedy)")
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--top-k", type=int, default=-1)
@@ -77,30 +230,40 @@ def main() -> int:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not built")
         return 2
 
+    import logging
+
     import torch
 
     from atom_amd import LLMEngine, SamplingParams
     from atom_amd.config import model_config_from_dict
 
-    raw = dict(QWEN3_8B)
+    logging.basicConfig(level=logging.INFO, stream=sys.stderr, format="[bench] %(name)s: %(message)s")
+    logging.getLogger("atom_amd").setLevel(logging.INFO if args.shape == "32b" else logging.WARNING)
+    name, shape, seed = SHAPES[args.shape]
+    raw = dict(shape)
     full_layers = raw["num_hidden_layers"]
     layers = args.layers or full_layers
     raw["num_hidden_layers"] = layers
     cfg = model_config_from_dict(raw)
+    mixed = args.mixed or (32 if args.shape == "4b" else 0)
+    long_run = args.shape == "32b" and not mixed
     points = sorted({int(x) for x in args.points.split(",") if x} | {args.batch})
-    points = [p for p in points]
-    max_seqs = max(points + [args.mixed])
-    max_model_len = args.max_model_len or max(4096, 2 * args.context)
     block = 16
+    if long_run:
+        max_seqs, max_model_len, pages, budget = 16, args.max_model_len or 8192 + 512, -1, 4096
+    else:
+        max_seqs = max(points + [mixed])
+        max_model_len = args.max_model_len or max(4096, 2 * args.context)
+        pages, budget = max_seqs * max_model_len // block, 16384
     t0 = time.time()
-    llm = LLMEngine("qwen3-8b-random", model_config=cfg, load_dummy="random", seed=2, dtype="bf16",
-                    max_model_len=max_model_len, kv_cache_block_size=block,
-                    num_kvcache_blocks=max_seqs * max_model_len // block, max_num_seqs=max_seqs,
-                    max_num_batched_tokens=16384, enforce_eager=args.enforce_eager,
-                    deferred_output=not args.no_deferred_output)
+    llm = LLMEngine(f"{name.lower()}-random", model_config=cfg, load_dummy="random", seed=seed, dtype="bf16",
+                    max_model_len=max_model_len, kv_cache_block_size=block, num_kvcache_blocks=pages,
+                    max_num_seqs=max_seqs, max_num_batched_tokens=budget, enforce_eager=args.enforce_eager,
+                    deferred_output=not args.no_deferred_output,
+                    cudagraph_capture_sizes=[s for s in (1, 2, 4, 8, 16, 32, 48, 64, 128, 256) if s <= max_seqs])
     torch.cuda.synchronize()
     print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
-    gen = torch.Generator().manual_seed(2)
+    gen = torch.Generator().manual_seed(seed)
     vocab = raw["vocab_size"]
 
     def prompt():
@@ -109,26 +272,11 @@ def main() -> int:
     def sync():
         torch.cuda.synchronize()
 
-    if args.mixed:
-        # continuous batching under load: every step holds the running requests' decode tokens and, under a
-        # budget of 512 + N tokens, the next portion of a waiting prompt
-        llm.scheduler.max_num_batched_tokens = 512 + args.mixed
-        lens = torch.randint(64, 3073, (args.mixed,), generator=gen).tolist()
-        sp = SamplingParams(temperature=0.0, max_tokens=128, ignore_eos=True)
-        prompts = [torch.randint(0, vocab, (n,), generator=gen).tolist() for n in lens]
-        sync()
-        t = time.perf_counter()
-        outs = llm.generate(prompts, sp)
-        sync()
-        elapsed = time.perf_counter() - t
-        assert all(o["num_tokens_output"] == 128 for o in outs)
-        print(json.dumps({"workload": "mixed", "requests": args.mixed, "prompt_tokens": sum(lens),
-                          "output_tokens": 128 * args.mixed, "seconds": round(elapsed, 3),
-                          "output_tok_s": round(128 * args.mixed / elapsed, 1),
-                          "total_tok_s": round((sum(lens) + 128 * args.mixed) / elapsed, 1),
-                          "steps": llm.core.steps_run, "preemptions": llm.scheduler.total_preemptions,
-                          "mean_ttft_ms": round(1e3 * sum(o["ttft"] for o in outs) / len(outs), 1),
-                          "mean_tpot_ms": round(1e3 * sum(o["tpot"] for o in outs) / len(outs), 2)}), flush=True)
+    if mixed:
+        print(json.dumps(run_mixed(llm, args, name, raw, layers, gen, mixed)), flush=True)
+        return 0
+    if long_run:
+        print(json.dumps(run_long(llm, args, name, raw, layers, gen)), flush=True)
         return 0
 
     # ---- prefill of one 2,048-token prompt
@@ -185,27 +333,29 @@ def main() -> int:
         print(f"[bench] decode batch {b}: {b * steps / elapsed:.1f} tok/s, {elapsed / steps * 1e3:.3f} ms/step",
               file=sys.stderr, flush=True)
 
+    def roofline(b):
+        elapsed, ctx0, steps = results[b]
+        step_bytes = weight_bytes(raw, layers) + b * (ctx0 + steps / 2) * kv_bytes_per_token(raw, layers)
+        return step_bytes * steps / elapsed
+
     elapsed, ctx0, steps = results[args.batch]
     per_step = elapsed / steps
-    mean_ctx = ctx0 + steps / 2
-    step_bytes = weight_bytes(raw, layers) + args.batch * mean_ctx * kv_bytes_per_token(raw, layers)
-    achieved = step_bytes / per_step
+    achieved = roofline(args.batch)
     line = {
-        "metric": "decode tok/s at batch 8 (Qwen3-8B, bf16); prefill tok/s at 2048 tokens and batch 1/64 alongside",
+        "metric": f"decode tok/s at batch {args.batch} ({name}, bf16); prefill tok/s at {args.context} tokens and "
+                  f"batch {'/'.join(str(b) for b in points if b != args.batch)} alongside",
         "value": round(args.batch * steps / elapsed, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
         "warmup": args.warmup, "ms_per_step": round(per_step * 1e3, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic: seeded uniform random token ids, seeded random N(0, 0.02) weights",
-        "config": {"model": "Qwen3-8B shape, random weights", "global_batch": args.batch, "seq_len": args.context,
-                   "parallelism": "single GPU", "layers": layers, "layers_of_model": full_layers,
-                   "hidden_size": raw["hidden_size"], "num_attention_heads": raw["num_attention_heads"],
-                   "num_key_value_heads": raw["num_key_value_heads"], "head_dim": raw["head_dim"],
-                   "intermediate_size": raw["intermediate_size"], "vocab_size": vocab,
-                   "max_model_len": max_model_len, "kv_block_size": block, "decode_steps": steps,
-                   "hip_graphs": not args.enforce_eager, "deferred_output": not args.no_deferred_output},
+        "config": flat_config(name, raw, layers, global_batch=args.batch, seq_len=args.context,
+                              max_model_len=max_model_len, decode_steps=steps, hip_graphs=not args.enforce_eager,
+                              deferred_output=not args.no_deferred_output),
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": {f"decode_b{b}": round(b * results[b][2] / results[b][0], 2) for b in points if b != args.batch},
+        # the same fraction of the HBM peak for the other batch sizes
+        "points_roofline": {f"decode_b{b}": round(roofline(b) / HBM_PEAK, 4) for b in points if b != args.batch},
     }
     if prefill:
         line["prefill"] = prefill

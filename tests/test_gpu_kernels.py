@@ -602,7 +602,11 @@ def _deferred(ops, m, n, k, seed, bias=True):
     x = rnd((m, k), torch.bfloat16, seed, 1.0)
     w = rnd((n, k), torch.bfloat16, seed + 1, 0.05)
     b = rnd((n,), torch.float32, seed + 2, 0.3) if bias else None
-    got = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV) if bias else None, defer=True)
+    ops.use_rows_gemm = False    # few rows would otherwise take the product that cuts nothing
+    try:
+        got = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV) if bias else None, defer=True)
+    finally:
+        ops.use_rows_gemm = True
     assert isinstance(got, DeferredSum) and got.splits > 1, "this shape was chosen so that K is cut"
     want = x.double() @ w.double().T + (b.double() if bias else 0)
     return got, want
@@ -666,3 +670,155 @@ def test_feed_tokens():
         want = torch.where(source >= 0, sampled[source.clamp(min=0).long()], ids)
         got = ops.feed_tokens(ids.cuda(), source.cuda(), sampled.cuda())
         assert torch.equal(got.cpu(), want)
+
+
+# ------------------------------------------------------------------ the few-rows product with norm and residual folded in
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 5, 8])
+@pytest.mark.parametrize("n,k", [(311, 136), (4096, 4096), (6144, 2560), (130, 12288), (16, 8), (1031, 520), (5000, 9728)])
+@pytest.mark.parametrize("waves", [0, 4, 8])
+def test_rows_product_plain_gate_and_residual(m, n, k, waves):
+    from atom_amd.kernels.hip import PendingNorm, PendingProduct
+
+    ops = gpu_ops()
+    ops.rows_waves = waves
+    try:
+        x = rnd((m, k), torch.bfloat16, 50, 1.0)
+        w = rnd((n, k), torch.bfloat16, 51, 0.05)
+        b = rnd((n,), torch.float32, 52, 0.5)
+        want = x.double() @ w.double().T + b.double()
+        scale = float(want.abs().max())
+        assert ops._rows_takes(x.to(DEV), w.to(DEV))
+        for out_dtype in (torch.bfloat16, torch.float32):
+            y = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), out_dtype=out_dtype)
+            assert y.dtype == out_dtype
+            close(y, want, torch.bfloat16, scale=scale)
+            if out_dtype == torch.float32:
+                assert float((y.cpu().double() - want).abs().max()) <= 1e-4 * scale
+                alone = ops.linear(x[m - 1:].to(DEV).contiguous(), w.to(DEV), b.to(DEV), out_dtype=out_dtype)
+                assert torch.equal(alone[0], y[m - 1]), "a row's sum does not depend on the rows beside it"
+        # deferred: nothing is launched until something wants it
+        pending = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), defer=True)
+        assert isinstance(pending, PendingProduct) and tuple(pending.shape) == (m, n)
+        close(ops.materialize(pending), want, torch.bfloat16, scale=scale)
+        # ... a norm with the residual stream makes it add in place and leaves the norm pending
+        res = rnd((m, n), torch.float32, 53, 2.0)
+        gamma = 1 + rnd((n,), torch.float32, 54, 0.2)
+        res_gpu = res.to(DEV)
+        lazy = ops.pending_norm(pending, res_gpu, gamma.to(DEV), 1e-5)
+        assert isinstance(lazy, PendingNorm) and lazy.r is res_gpu
+        new_res = res.double() + want
+        assert float((res_gpu.cpu().double() - new_res).abs().max()) <= 1e-4 * float(new_res.abs().max())
+        ss_want = new_res.pow(2).sum(-1)
+        assert torch.allclose(lazy.ss.sum(-1).cpu().double(), ss_want, rtol=1e-5)
+        normed_want = new_res * torch.rsqrt(new_res.pow(2).mean(-1, keepdim=True) + 1e-5) * gamma.double()
+        close(ops.materialize(lazy), normed_want, torch.bfloat16)
+        # ... which the next product applies while it reads (here: back down to a width of 200, and SiLU-gated)
+        if n % 8 == 0:
+            w2 = rnd((200, n), torch.bfloat16, 55, 0.05)
+            xn = normed_want.to(torch.bfloat16).double()
+            y2 = ops.linear(lazy, w2.to(DEV), None, out_dtype=torch.float32)
+            want2 = xn @ w2.double().T
+            assert float((y2.cpu().double() - want2).abs().max()) <= 1.2e-2 * float(want2.abs().max())
+            wg = rnd((2 * 104, n), torch.bfloat16, 56, 0.05)
+            bg = rnd((2 * 104,), torch.float32, 57, 0.3)
+            act = ops.linear_silu(lazy, wg.to(DEV), bg.to(DEV))
+            gu = xn @ wg.double().T + bg.double()
+            want_act = torch.nn.functional.silu(gu[:, :104]) * gu[:, 104:]
+            close(act, want_act, torch.bfloat16)
+            # ... also at chosen rows only (the head of a step that wants some rows' logits)
+            if m >= 3:
+                pick = torch.tensor([m - 1, 0], dtype=torch.int32, device=DEV)
+                picked = PendingNorm(lazy.r, lazy.xg, lazy.ss, lazy.weight, lazy.eps, pick, lazy.dtype)
+                y3 = ops.linear(picked, w2.to(DEV), None, out_dtype=torch.float32)
+                assert torch.equal(y3[0], y2[m - 1]) and torch.equal(y3[1], y2[0])
+    finally:
+        ops.rows_waves = 0
+
+
+def test_rows_product_gate_alone_and_odd_widths():
+    ops = gpu_ops()
+    for m, inter, k in [(1, 200, 136), (8, 12288, 4096), (4, 333, 264), (7, 9, 40)]:
+        x = rnd((m, k), torch.bfloat16, 60, 1.0)
+        w = rnd((2 * inter, k), torch.bfloat16, 61, 0.05)
+        b = rnd((2 * inter,), torch.float32, 62, 0.3)
+        gu = x.double() @ w.double().T + b.double()
+        want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+        close(ops.linear_silu(x.to(DEV), w.to(DEV), b.to(DEV)), want, torch.bfloat16)
+
+
+# ------------------------------------------------------------------ decode attention that starts from the QKV product
+
+
+@pytest.mark.parametrize("hq,hkv,d,page", [(32, 8, 128, 16), (8, 2, 64, 8), (6, 3, 64, 16), (4, 1, 256, 32), (40, 2, 128, 16)])
+@pytest.mark.parametrize("norm", [True, False])
+@pytest.mark.parametrize("window", [None, 40])
+def test_fused_decode_attention_matches_the_separate_kernels(hq, hkv, d, page, norm, window):
+    """Per-head norm, rotation, cache write and attention in one kernel against the same step as two kernels,
+    for requests whose new token is the first of a page, the last, in the middle, and a padding row."""
+    from atom_amd.kernels.hip import PendingProduct
+
+    ops = gpu_ops()
+    ctxs = [1, page, page + 1, 5 * page - 1, 333, 0, 97]       # keys of each request with the new token; 0: padding
+    seqs, hidden = len(ctxs), 264
+    width = -(-max(ctxs) // page)
+    pages = seqs * width + 1
+    g = torch.Generator().manual_seed(7)
+    tables = torch.randperm(pages - 1, generator=g)[:seqs * width].view(seqs, width).to(torch.int32) + 1
+    x = rnd((seqs, hidden), torch.bfloat16, 90)
+    w = rnd(((hq + 2 * hkv) * d, hidden), torch.bfloat16, 91, 0.1)
+    b = rnd(((hq + 2 * hkv) * d,), torch.float32, 92, 0.3)
+    qw = (1 + rnd((d,), torch.float32, 93, 0.2)).to(DEV) if norm else None
+    kw = (1 + rnd((d,), torch.float32, 94, 0.2)).to(DEV) if norm else None
+    inv = 1.0 / (10000.0 ** (torch.arange(0, d, 2).float() / d))
+    ang = torch.arange(512).float()[:, None] * inv[None, :]
+    cos, sin = ang.cos().to(DEV), ang.sin().to(DEV)
+    k0 = rnd((pages, hkv, page, d), torch.bfloat16, 95)
+    v0 = rnd((pages, hkv, d, page), torch.bfloat16, 96)
+    pos = torch.tensor([max(c - 1, 0) for c in ctxs], dtype=torch.int32)
+    slots = torch.tensor([int(tables[s, (c - 1) // page]) * page + (c - 1) % page if c else -1 for s, c in enumerate(ctxs)],
+                         dtype=torch.int32)
+    meta = AttentionMeta(token_seq=torch.tensor([s if c else -1 for s, c in enumerate(ctxs)], dtype=torch.int32).to(DEV),
+                         positions=pos.to(DEV), block_tables=tables.to(DEV).contiguous(),
+                         cu_seqlens_q=torch.arange(seqs + 1, dtype=torch.int32).to(DEV),
+                         context_lens=torch.tensor(ctxs, dtype=torch.int32).to(DEV), num_seqs=seqs, num_tokens=seqs,
+                         max_q_len=1, max_context_len=max(ctxs), page_size=page, num_prefill=0)
+
+    def pending():
+        got = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), defer=True)
+        assert isinstance(got, PendingProduct)
+        return got
+
+    results = []
+    for fused in (True, False):
+        kc, vc = k0.clone().to(DEV), v0.clone().to(DEV)
+        out = torch.full((seqs, hq, d), float("nan"), dtype=torch.bfloat16, device=DEV)
+        for parts in (1, 4, 13):
+            if fused:
+                done = ops.fused_decode_attention(pending(), kc, vc, out, meta, d ** -0.5, window, qw, kw, cos, sin,
+                                                  slots.to(DEV), hq, hkv, d, d, 1e-5, parts=parts)
+                assert done is out
+            else:
+                q = torch.empty((seqs, hq, d), dtype=torch.bfloat16, device=DEV)
+                ops.qk_norm_rope_kv_write(pending(), q, kc, vc, qw, kw, cos, sin, pos.to(DEV), slots.to(DEV), hq, hkv, d, d,
+                                          page, 1e-5)
+                ops.paged_attention(q, kc, vc, out, meta, d ** -0.5, window, parts=parts)
+            results.append((fused, parts, out.clone().cpu(), kc.cpu().clone(), vc.cpu().clone()))
+    want = {parts: r for f, parts, *r in results if not f}
+    for f, parts, out, kc, vc in results:
+        if not f:
+            continue
+        ref_out, ref_k, ref_v = want[parts]
+        assert torch.equal(vc, ref_v), "the new values land in the same places"
+        assert float((kc.float() - ref_k.float()).abs().max()) <= 2e-2 * float(ref_k.float().abs().max())
+        assert (kc != ref_k).float().mean() < 1e-3, "only the new keys may differ, and only by a rounding"
+        live = [s for s, c in enumerate(ctxs) if c]
+        close(out[live], ref_out[live].double(), torch.bfloat16)
+        assert float(out[ctxs.index(0)].float().abs().max()) == 0.0, "a padding row attends to nothing"
+    # a layer that reads another layer's cache writes nothing
+    kc, vc = k0.clone().to(DEV), v0.clone().to(DEV)
+    out = torch.empty((seqs, hq, d), dtype=torch.bfloat16, device=DEV)
+    ops.fused_decode_attention(pending(), kc, vc, out, meta, d ** -0.5, window, qw, kw, cos, sin, None, hq, hkv, d, d,
+                               1e-5, write_kv=False)
+    assert torch.equal(kc.cpu(), k0) and torch.equal(vc.cpu(), v0)

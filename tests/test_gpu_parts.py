@@ -153,7 +153,7 @@ def test_gated_mlp_part(dtype):
     x = rnd((3, 96), 6).to(dtype)
     gu = w["m.gate_up.weight"]
     want = pm.gated_mlp(x.double(), gu[:160], gu[160:], w["m.down.weight"])
-    check(mlp.forward(ctx, x.to(DEV)), want, dtype)
+    check(gpu_ops().materialize(mlp.forward(ctx, x.to(DEV))), want, dtype)   # few rows: the down product is still pending
     with pytest.raises(ValueError):
         GatedMLP(8, 8, activation="gelu")
 
