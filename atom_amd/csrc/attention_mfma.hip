@@ -98,6 +98,7 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
   } else {
     const int tile = blockIdx.x;
     seq = p.tiles[2 * tile];
+    if (seq < 0) return;   // an unused entry of a list of fixed length
     const int row_start = p.tiles[2 * tile + 1];
     head0 = blockIdx.y;
     kvh = head0 / group;
@@ -845,6 +846,7 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
     ygroup = blockIdx.y;
   }
   const int seq = p.tiles[2 * tile];
+  if (seq < 0) continue;   // an unused entry of a list of fixed length (the same for the whole block)
   const int row_start = p.tiles[2 * tile + 1];
   const int head = ygroup * GH + (wave % GH);
   const int kvh = (ygroup * GH) / group;

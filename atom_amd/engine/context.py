@@ -26,9 +26,23 @@ class BatchView:
     cached: list[int]              # tokens of each request before this step
     num_prefill: int               # how many requests bring more than one token
     page_sizes: list[int]          # of each group of layers
-    # the step is (or will be) replayed from a captured graph: rows beyond the live requests are padding
-    # with one token and no context, and the arrays' shapes may depend on ``q_lens`` only
+    # The step is (or will be) replayed from a captured graph: the arrays' shapes may depend only on the
+    # number of requests and on the two capacities below.  Request rows without a live request are padding:
+    # single-token rows with no context, and, where prompt portions are held, one row behind the
+    # ``prefill_slots`` portion rows that owns the unused token rows (it counts in ``num_prefill``; a portion
+    # row that is not in use has no tokens).
     replayed: bool = False
+    prefill_capacity: int = 0      # replayed: token rows set aside for prompt portions
+    prefill_slots: int = 0         # replayed: request rows set aside for prompt portions
+
+    def portions(self) -> list[int]:
+        """The request rows that bring a prompt portion in this step."""
+        rows = range(self.prefill_slots) if self.replayed else range(self.num_prefill)
+        return [b for b in rows if self.q_lens[b] > 1]
+
+    def tile_capacity(self, rows: int) -> int:
+        """How many tiles of ``rows`` query rows the portions of a replayed step can need at most."""
+        return -(-self.prefill_capacity // rows) + self.prefill_slots
 
     @property
     def num_seqs(self) -> int:
@@ -36,6 +50,9 @@ class BatchView:
 
     @property
     def max_q_len(self) -> int:
+        """The most tokens a request brings (in a replayed step: can bring)."""
+        if self.replayed:
+            return max(self.prefill_capacity, 1)
         return max(self.q_lens) if self.q_lens else 0
 
 

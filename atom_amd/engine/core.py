@@ -42,7 +42,8 @@ class StepEntry:
 
 class EngineCore:
     def __init__(self, model, ops, plan: CachePlan, max_num_seqs: int, device, dtype: torch.dtype,
-                 graph_sizes: list[int] | None = None, max_model_len: int = 0, prefix_caching: bool = False):
+                 graph_sizes: list[int] | None = None, max_model_len: int = 0, prefix_caching: bool = False,
+                 graph_prefill_sizes: list[int] | None = None):
         self.model = model
         self.ops = ops
         self.device = torch.device(device)
@@ -73,7 +74,7 @@ class EngineCore:
         if graph_sizes:
             from .graphs import DecodeGraphs
 
-            graphs = DecodeGraphs(self, graph_sizes, max_model_len or self.max_positions)
+            graphs = DecodeGraphs(self, graph_sizes, max_model_len or self.max_positions, graph_prefill_sizes)
             self.graphs = graphs if graphs.usable else None
 
     # ------------------------------------------------------------------ requests
@@ -158,14 +159,7 @@ class EngineCore:
 
         cached_now = [self.lengths[e.req_id] for e in entries]
         if self.graphs is not None and self.graphs.accepts(entries, cached_now):
-            rows = [b for b, e in enumerate(entries) if e.want]
-            logits = None
-            all_logits = self.graphs.run(entries, cached_now)
-            if len(rows) == len(entries):
-                logits = all_logits          # every row wanted: the graph's own output, valid until its next replay
-            elif rows:
-                index = torch.tensor(rows, dtype=torch.long, device=self.device)
-                logits = all_logits.index_select(0, index)
+            logits = self.graphs.run(entries, cached_now)
         else:
             ctx, token_ids, want_rows = self._build(entries, order)
             logits = self.model.forward(ctx, token_ids, self.storage.bindings, want_rows)
@@ -183,10 +177,12 @@ class EngineCore:
         if req_id in self.lengths and self.manager.awaited_position(req_id) == position:
             self.manager.amend(req_id, position, token)
 
-    def batch_view(self, q_lens: list[int], cached: list[int], replayed: bool = False) -> BatchView:
+    def batch_view(self, q_lens: list[int], cached: list[int], replayed: bool = False, prefill_capacity: int = 0,
+                   prefill_slots: int = 0, num_prefill: int | None = None) -> BatchView:
         return BatchView(ops=self.ops, dtype=self.dtype, q_lens=q_lens, cached=cached,
-                         num_prefill=sum(1 for n in q_lens if n > 1),
-                         page_sizes=[g.page_size for g in self.manager.groups], replayed=replayed)
+                         num_prefill=sum(1 for n in q_lens if n > 1) if num_prefill is None else num_prefill,
+                         page_sizes=[g.page_size for g in self.manager.groups], replayed=replayed,
+                         prefill_capacity=prefill_capacity, prefill_slots=prefill_slots)
 
     def _build(self, entries: list[StepEntry], order: list[int]):
         """Every array of the step in one int32 host buffer (pinned), one copy to the device, and the
@@ -329,11 +325,12 @@ def load_model(model_dir: str | None, *, dtype: torch.dtype, device, model_confi
 def build_core(model, ops, *, dtype: torch.dtype, device, page_size: int = 16, num_pages: int | None = None,
                budget_bytes: int | None = None, max_num_seqs: int = 4, max_model_len: int = 0,
                max_num_batched_tokens: int = 0, graph_sizes: list[int] | None = None,
-               prefix_caching: bool = False) -> EngineCore:
+               prefix_caching: bool = False, graph_prefill_sizes: list[int] | None = None) -> EngineCore:
     from ..cache.storage import plan_cache
 
     plan = plan_cache(model, page_size, dtype, num_pages=num_pages, budget_bytes=budget_bytes,
                       max_num_seqs=max_num_seqs, max_model_len=max_model_len,
                       max_num_batched_tokens=max_num_batched_tokens)
     return EngineCore(model, ops, plan, max_num_seqs, device, dtype, graph_sizes=graph_sizes,
-                      max_model_len=max_model_len, prefix_caching=prefix_caching)
+                      max_model_len=max_model_len, prefix_caching=prefix_caching,
+                      graph_prefill_sizes=graph_prefill_sizes)

@@ -101,7 +101,7 @@ class LLMEngine:
             max_num_seqs=cfg.max_num_seqs, max_model_len=cfg.max_model_len,
             max_num_batched_tokens=cfg.max_num_batched_tokens,
             graph_sizes=None if cfg.enforce_eager else cfg.cudagraph_capture_sizes,
-            prefix_caching=cfg.enable_prefix_caching)
+            graph_prefill_sizes=cfg.cudagraph_prefill_sizes, prefix_caching=cfg.enable_prefix_caching)
         self._log_capacity()
         if self.core.graphs is not None:   # as the reference's engine does before it serves (engine_core.py:131-138)
             captured = self.core.graphs.capture_all()

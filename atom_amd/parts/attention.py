@@ -82,15 +82,19 @@ class GroupedQueryAttention(Mixer):
 
     def prepare_step(self, batch) -> dict:
         """Tiles of query rows of the prompt portions, as (request, first row) pairs, the tiles with the most
-        keys first: one list for every tile height the kernels of this step use."""
+        keys first: one list for every tile height the kernels of this step use.  In a replayed step every
+        list has the length the bucket can need at most; entries beyond the step's tiles name request -1."""
         if not batch.num_prefill:
             return {}
         out = {}
+        portions = batch.portions()
         for page_size in set(batch.page_sizes):
             for rows in self._tile_rows(batch.ops, batch.dtype, page_size, batch.max_q_len):
                 if rows and f"tiles{rows}" not in out:
-                    tiles = [(b, r0) for b in range(batch.num_prefill) for r0 in range(0, batch.q_lens[b], rows)]
+                    tiles = [(b, r0) for b in portions for r0 in range(0, batch.q_lens[b], rows)]
                     tiles.sort(key=lambda t: -(batch.cached[t[0]] + t[1]))
+                    if batch.replayed:
+                        tiles += [(-1, 0)] * (batch.tile_capacity(rows) - len(tiles))
                     out[f"tiles{rows}"] = np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
         return out
 

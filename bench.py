@@ -116,7 +116,6 @@ def run_mixed(llm, args, name, raw, layers, gen, requests: int) -> dict:
     from atom_amd import SamplingParams
 
     vocab = raw["vocab_size"]
-    llm.scheduler.max_num_batched_tokens = 512 + requests
     sp = SamplingParams(temperature=0.0, max_tokens=128, ignore_eos=True)
     warm = [torch.randint(0, vocab, (n,), generator=gen).tolist() for n in (700, 90)]
     llm.generate(warm, SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))   # untimed: first-use work
@@ -254,7 +253,7 @@ def main() -> int:
     else:
         max_seqs = max(points + [mixed])
         max_model_len = args.max_model_len or max(4096, 2 * args.context)
-        pages, budget = max_seqs * max_model_len // block, 16384
+        pages, budget = max_seqs * max_model_len // block, (512 + mixed if mixed else 16384)
     t0 = time.time()
     llm = LLMEngine(f"{name.lower()}-random", model_config=cfg, load_dummy="random", seed=seed, dtype="bf16",
                     max_model_len=max_model_len, kv_cache_block_size=block, num_kvcache_blocks=pages,

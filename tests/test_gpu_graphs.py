@@ -34,6 +34,37 @@ def test_graph_cuts_match_plain(which, cut, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["B", "C", "D"])
+def test_steps_with_prompt_portions_replayed_as_graphs(which, dtype):
+    """Steps as a scheduler under a small budget makes them (one or two prompt portions beside single tokens)
+    run as replayed graphs of fixed shape, padded in both parts, and give the plain implementation's logits."""
+    lengths = {"B": [30, 71, 200, 130, 12, 90], "C": [50, 400, 95, 257, 31, 140], "D": [45, 300, 130, 260, 20]}[which]
+    requests = {f"m{k}": random_ids(which, n, 500 + k) for k, n in enumerate(lengths)}
+    oracle = {rid: oracle_logits(which, ids) for rid, ids in requests.items()}
+    steps = replay.scheduled(requests, seed=3, max_live=4, budget=100)
+    pages = -(-replay.peak_tokens(steps, 64) // 16)
+    from atom_amd.engine.core import TORCH_DTYPES, build_core, load_model
+    from helpers import tiny_folder
+
+    model, _ = load_model(tiny_folder(which), dtype=TORCH_DTYPES[dtype], device="cuda:0")
+    core = build_core(model, gpu_ops(), dtype=TORCH_DTYPES[dtype], device="cuda:0", page_size=16, num_pages=pages,
+                      max_num_seqs=8, graph_sizes=[1, 2, 4, 8], graph_prefill_sizes=[48, 128])
+    results = replay.run_in_process(core, steps)
+    mixed = sum(1 for s in steps if any(len(e["tokens"]) > 1 for e in s["entries"]))
+    assert mixed >= 6 and core.graphs.mixed_replays == mixed, "every step with a prompt portion fits a bucket here"
+    assert {shape[0] for shape in core.graphs.captured} >= {0, 48, 128}
+    replay.check(steps, results, requests, oracle, dtype, f"mixed graph/{which}/{dtype}", every=False)
+    # the same steps eagerly: the same logits within rounding
+    eager = build_core(model, gpu_ops(), dtype=TORCH_DTYPES[dtype], device="cuda:0", page_size=16, num_pages=pages,
+                       max_num_seqs=8)
+    plain = replay.run_in_process(eager, steps)
+    tol = (1e-5 if dtype == "float32" else 3e-2)
+    for k in results:
+        scale = float(plain[k].abs().max())
+        assert float((results[k] - plain[k]).abs().max()) <= tol * scale, f"step {k}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("live,bucket", [(3, 4), (27, 32)])
 def test_replays_agree_with_eager(dtype, live, bucket):
     """Requests decode together through one graph (with padding rows) for 12 steps; in between, another
