@@ -31,9 +31,10 @@ class Config:
     deferred_output: bool = True
     cudagraph_capture_sizes: list[int] = field(default_factory=lambda: [1, 2, 4, 8, 16, 32, 48, 64, 128, 256])
     # Steps that hold prompt portions beside decode tokens are replayed as graphs too when the portions
-    # together have at most this many tokens (one graph per listed size and decode size).  None: [128, 512]
-    # when the token budget is small enough for such steps to be the usual ones (at most 2,048), else none.
-    cudagraph_prefill_sizes: list[int] | None = None
+    # together have at most one of these many tokens (one graph per listed size and decode size of 8 and more).
+    # Off by default: on an MI355X such steps keep the GPU busy when launched one by one, as long as they are
+    # launched ahead (deferred_output), and a graph pads every step to its bucket.
+    cudagraph_prefill_sizes: list[int] = field(default_factory=list)
     hf_overrides: dict | None = None
     dtype: str = "bf16"
     seed: int = 0
@@ -69,8 +70,6 @@ class Config:
                 raise ConfigError("long_prefill_token_threshold must not exceed max_model_len")
             if self.long_prefill_token_threshold < self.kv_cache_block_size:
                 raise ConfigError("long_prefill_token_threshold must be at least one cache block")
-        if self.cudagraph_prefill_sizes is None:
-            self.cudagraph_prefill_sizes = [128, 512] if self.max_num_batched_tokens <= 2048 else []
         if self.max_num_seqs <= 0 or self.max_num_batched_tokens <= 0:
             raise ConfigError("max_num_seqs and max_num_batched_tokens must be positive")
         if not (0.0 < self.gpu_memory_utilization <= 1.0):

@@ -112,6 +112,8 @@ class LLMEngine:
         self._profiler = None
         self.deferred_output = bool(cfg.deferred_output)
         self._in_flight: _InFlight | None = None
+        self.steps_launched = 0          # steps queued on the device so far ...
+        self.steps_launched_ahead = 0    # ... and how many of them before the step before them had been read
         # two pinned buffers take turns: a step's tokens are read while the next step's are on their way
         self._stages = [_Stage(cfg.max_num_seqs, pinned=torch.device(cfg.device).type == "cuda") for _ in range(2)]
         self._next_stage = 0
@@ -225,6 +227,7 @@ class LLMEngine:
             batch = self.scheduler.schedule_ahead(running.batch)
             if batch is not None:
                 ahead = self._launch(batch, {it.seq.id: k for k, it in enumerate(running.finals)})
+                self.steps_launched_ahead += 1
         done += self._finish(running)
         self._in_flight = ahead
         return done
@@ -232,6 +235,7 @@ class LLMEngine:
     def _launch(self, batch, sampled_rows: dict[int, int] | None) -> "_InFlight":
         """Queues the batch's step and its sampling on the device; waits for nothing."""
         start = time.time()
+        self.steps_launched += 1
         with torch.profiler.record_function(self._run_label(batch)):
             logits = self.core.step(batch.entries(sampled_rows))
         finals = [it for it in batch.items if it.is_final]

@@ -91,6 +91,8 @@ class Scheduler:
         self.total_preemptions = 0
         self._last_prompt_time = 0.0
         self._last_prompt_latency = 0.0
+        # requests that reach their token count in the step that is still running: a step scheduled ahead leaves them out
+        self._sit_out: set[int] = set()
 
     # ------------------------------------------------------------------ queues
 
@@ -241,7 +243,8 @@ class Scheduler:
         # ---- running requests that decode: one token each
         for seq in list(self.running):
             # a request preempted earlier in this loop is WAITING by now
-            if seq.status != SequenceStatus.RUNNING or seq.is_partial_prefill or seq.id in scheduled:
+            if (seq.status != SequenceStatus.RUNNING or seq.is_partial_prefill or seq.id in scheduled
+                    or seq.id in self._sit_out):
                 continue
             if len(batch.items) >= self.max_num_seqs or batched + 1 > self.max_num_batched_tokens:
                 break
@@ -331,48 +334,59 @@ class Scheduler:
 
     def schedule_ahead(self, running_batch: ScheduledBatch) -> ScheduledBatch | None:
         """The batch that follows ``running_batch``, made before that batch's tokens are known, so that
-        the device never waits for the host between two decode steps (the reference's deferred output,
-        atom/model_engine/model_runner.py:358-392, scheduler.py:2127-2133).  Only the steady case is taken:
-        every running request is in ``running_batch`` and gets a token from it, nothing can be admitted
-        (now, or because a request reaches its token count in ``running_batch``), and the pools hold
-        the pages of one more token for all of them.  Every request of
-        ``running_batch`` then ends in a placeholder, and those that cannot finish by their token
-        count decode once more.  In every other case this returns None and changes nothing: the caller
-        waits for the running batch and schedules as usual."""
-        if self._rejected or (self.waiting and len(self.running) < self.max_num_seqs):
+        the device never waits for the host between two steps (the reference's deferred output,
+        atom/model_engine/model_runner.py:358-392, scheduler.py:2127-2133).
+
+        What ``running_batch`` does to its requests apart from the tokens' values is applied at once: their
+        cached lengths move on, and every request that gets a token from it ends in a placeholder until the
+        token arrives.  Then the ordinary ``schedule`` makes the next batch: decode tokens (read on the device
+        from the sampler's output), further prompt portions, admissions.  This is done only when nothing in it
+        can depend on the tokens' values: no request reaches its token count in ``running_batch`` while others
+        wait for its place (with nobody waiting such a request simply takes no further part), and the pools hold
+        the pages of one more token for every decoding request, so that nobody has to be preempted.  A request
+        that turns out to have ended on its token (eos, a stop sequence) has then run once too often, and that
+        result is dropped.  In every other case this returns None and changes nothing: the caller waits for
+        the running batch and schedules as usual."""
+        items = running_batch.items
+        if self._rejected or not items:
             return None
-        if len(running_batch.items) != len(self.running):
+        if any(it.seq.status != SequenceStatus.RUNNING or it.seq.awaits_token for it in items):
             return None
-        if any(not it.is_final or it.seq.status != SequenceStatus.RUNNING or it.seq.awaits_token
-               for it in running_batch.items):
+        if any(s.status != SequenceStatus.RUNNING or s.awaits_token for s in self.running):
             return None
         mgr = self.manager
-        plan = []
         need = [0] * len(mgr.groups)
-        for it in running_batch.items:
+        done_by_count = set()
+        for it in items:
+            if not it.is_final:
+                continue
             seq = it.seq
             # with the token that the running batch gives it
             if seq.num_completion_tokens + 1 >= seq.max_tokens or seq.num_tokens + 1 >= self.max_model_len:
                 if self.waiting:
                     return None   # its place goes to a waiting request in the very next step
+                done_by_count.add(seq.id)
                 continue
             after = it.start + it.num_tokens
             for gi, n in enumerate(mgr.pages_missing(seq.id, after, after + 1)):
                 need[gi] += n
-            plan.append((seq, after))
-        if not plan or len(plan) > min(self.max_num_seqs, self.max_num_batched_tokens):
-            return None
+        in_batch = {it.seq.id for it in items}
+        for seq in self.running:   # decoding requests that sat this batch out
+            if seq.id not in in_batch and not seq.is_partial_prefill:
+                for gi, n in enumerate(mgr.pages_missing(seq.id, seq.num_cached_tokens, seq.num_cached_tokens + 1)):
+                    need[gi] += n
         if any(n > mgr.num_free_pages(gi) for gi, n in enumerate(need)):
             return None
-        for it in running_batch.items:
+        for it in items:
             it.seq.num_cached_tokens = it.start + it.num_tokens
-            it.seq.is_partial_prefill = False
-            it.seq.append_placeholder()
-        batch = ScheduledBatch()
-        for seq, after in plan:
-            mgr.cover(seq.id, after, after + 1)
-            batch.items.append(ScheduledItem(seq, 1, after, True, True))
-        return batch
+            it.seq.is_partial_prefill = not it.is_final
+            if it.is_final:
+                it.seq.append_placeholder()
+        self._sit_out = done_by_count
+        try:
+            return self.schedule()
+        finally:
+            self._sit_out = set()
 
     # ------------------------------------------------------------------ after the step
 

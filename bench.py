@@ -142,7 +142,8 @@ def run_mixed(llm, args, name, raw, layers, gen, requests: int) -> dict:
                      "unit": "GB/s", "frac": round(counter.bytes / elapsed / HBM_PEAK, 4)},
         "mfma_frac": round(counter.flops / elapsed / MFMA_PEAK["bf16"], 4),
         "total_tok_s": round((sum(lens) + out_tokens) / elapsed, 1), "seconds": round(elapsed, 3),
-        "preemptions": llm.scheduler.total_preemptions,
+        "preemptions": llm.scheduler.total_preemptions, "steps_launched_ahead": llm.steps_launched_ahead,
+        "graph_replays": llm.core.graphs.replays if llm.core.graphs else 0,
         "mean_ttft_ms": round(1e3 * sum(o["ttft"] for o in outs) / len(outs), 1),
         "mean_tpot_ms": round(1e3 * sum(o["tpot"] for o in outs) / len(outs), 2),
     }

@@ -291,14 +291,14 @@ def test_default_cache_sizing_fills_the_allowed_memory_and_generates():
     want_pool = 4 << 30
     util = min(1.0, (total - free + int(total * 0.02) + want_pool + (1 << 30)) / total)
     llm = LLMEngine(tiny_folder("D"), dtype="bf16", ops=gpu_ops(), gpu_memory_utilization=util, max_num_seqs=8,
-                    max_model_len=512, cudagraph_capture_sizes=[1, 2, 4, 8])
+                    max_model_len=512, cudagraph_capture_sizes=[1, 2, 4, 8], cudagraph_prefill_sizes=[])
     plan = llm.core.plan
     assert llm.config.num_kvcache_blocks == -1 and llm.config.kv_cache_block_size == 16
     assert plan.groups[0].num_pages > 8 * 512 // 16, "the pool must hold more than every slot's longest request"
     assert 0.7 * want_pool <= plan.total_bytes() <= want_pool + (1 << 30)
     free_after, _ = torch.cuda.mem_get_info()
     assert total - free_after <= util * total, "weights, cache and graphs stay inside the allowed share"
-    assert llm.core.graphs is not None and sorted(llm.core.graphs.captured) == [1, 2, 4, 8]
+    assert llm.core.graphs is not None and sorted(llm.core.graphs.captured) == [(0, 0, n) for n in (1, 2, 4, 8)]
     prompts = [random_ids("D", n, 60 + n) for n in (5, 90, 33)]
     outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))
     assert llm.core.graphs.replays > 0

@@ -394,25 +394,66 @@ def test_schedule_ahead_skips_a_request_at_its_last_token():
     core.manager.check()
 
 
-def test_schedule_ahead_declines_and_changes_nothing():
-    # a request waits and could be admitted
+def test_schedule_ahead_admits_and_continues_prompts():
+    """What a step scheduled ahead may hold besides decode tokens: a request admitted meanwhile, the next
+    portion of an unfinished prompt; a prompt that ends in the running batch decodes in the next."""
     sched, core = make(blocks=40, block=4)
     a, = _decoding(sched, [6], max_tokens=9)
     running = sched.schedule()
-    sched.add(seq(range(50, 55)))                   # arrives while the batch runs
-    assert sched.schedule_ahead(running) is None and not a.awaits_token
-    # a prompt that ends in the running batch decodes in the next: its first token too is read on the device
-    sched.postprocess(running, {a.id: 5})
-    running = sched.schedule()
-    assert [it.is_decode for it in running.items] == [True, False]
+    new = seq(range(50, 55))
+    sched.add(new)                                  # arrives while the batch runs
     ahead = sched.schedule_ahead(running)
-    assert [(it.start, it.is_decode) for it in ahead.items] == [(8, True), (5, True)]
-    # ... but a full house keeps the waiting request out, so decoding runs ahead
+    assert [(it.seq.id, it.start, it.num_tokens, it.is_decode) for it in ahead.items] == [(a.id, 7, 1, True), (new.id, 0, 5, False)]
+    assert a.awaits_token and not new.awaits_token
+    entries = ahead.entries({a.id: 0})
+    assert [(e.tokens, e.feed) for e in entries] == [([Sequence.PLACEHOLDER], 0), (list(range(50, 55)), None)]
+    sched.postprocess(running, {a.id: 5})
+    assert a.token_ids[-1] == 5 and not a.awaits_token
+    # the prompt ended in the batch that is now running: its first token too is read on the device
+    running = ahead
+    ahead = sched.schedule_ahead(running)
+    assert [(it.seq.id, it.start, it.is_decode) for it in ahead.items] == [(a.id, 8, True), (new.id, 5, True)]
+    assert ahead.entries({a.id: 0, new.id: 1})[1].feed == 1
+    sched.postprocess(running, {a.id: 6, new.id: 7})
+    sched.postprocess(ahead, {a.id: 8, new.id: 9})
+    assert a.token_ids[-3:] == [5, 6, 8] and new.token_ids[-2:] == [7, 9]
+    core.manager.check()
+    # an unfinished prompt goes on with its next portion, beside a request that decodes
+    sched, core = make(blocks=100, block=4, max_num_batched_tokens=65)
+    d, = _decoding(sched, [6], max_tokens=9, ignore_eos=True)
+    long = seq(range(150))
+    sched.add(long)
+    running = sched.schedule()
+    assert [(it.num_tokens, it.is_final) for it in running.items] == [(1, True), (64, False)]
+    ahead = sched.schedule_ahead(running)
+    assert [(it.seq.id, it.start, it.num_tokens, it.is_final) for it in ahead.items] == [(d.id, 7, 1, True), (long.id, 64, 64, False)]
+    assert d.awaits_token and long.is_partial_prefill and not long.awaits_token and long.num_cached_tokens == 64
+    sched.postprocess(running, {d.id: 4})
+    third = sched.schedule_ahead(ahead)
+    assert [(it.start, it.num_tokens, it.is_final) for it in third.items] == [(8, 1, True), (128, 22, True)]
+    sched.postprocess(ahead, {d.id: 4})
+    sched.postprocess(third, {d.id: 4, long.id: 3})
+    assert long.num_completion_tokens == 1 and long.num_cached_tokens == 150
+    core.manager.check()
+
+
+def test_schedule_ahead_declines_and_changes_nothing():
+    # a request reaches its token count in the running batch while another waits for its place
+    sched, core = make(blocks=40, block=4, max_num_seqs=2)
+    a, b = _decoding(sched, [6, 7], max_tokens=9)
+    a.max_tokens = 2
+    sched.add(seq(range(50, 55)))
+    running = sched.schedule()
+    before = (a.num_tokens, b.num_tokens, b.num_cached_tokens, core.manager.num_free_pages(0))
+    assert sched.schedule_ahead(running) is None
+    assert (a.num_tokens, b.num_tokens, b.num_cached_tokens, core.manager.num_free_pages(0)) == before
+    assert not a.awaits_token and not b.awaits_token
+    # ... but a full house whose requests all go on keeps the waiting request out, so decoding runs ahead
     sched, core = make(blocks=40, block=4, max_num_seqs=2)
     a, b = _decoding(sched, [6, 7], max_tokens=9)
     sched.add(seq(range(50, 55)))
     running = sched.schedule()
-    assert sched.schedule_ahead(running) is not None
+    assert [it.is_decode for it in sched.schedule_ahead(running).items] == [True, True]
     # no page for the next token: left to the ordinary path, which preempts
     sched, core = make(blocks=4, block=4)
     a, b = _decoding(sched, [7, 7], max_tokens=9, ignore_eos=True)
@@ -420,11 +461,12 @@ def test_schedule_ahead_declines_and_changes_nothing():
     before = (a.num_tokens, a.num_cached_tokens, core.manager.num_free_pages(0))
     assert sched.schedule_ahead(running) is None
     assert (a.num_tokens, a.num_cached_tokens, core.manager.num_free_pages(0)) == before and not a.awaits_token
-    # an unfinished prompt in the running batch
-    sched, core = make(blocks=100, block=4, max_num_batched_tokens=64)
-    sched.add(seq(range(100)))
+    # a request of the running batch was aborted meanwhile
+    sched, core = make(blocks=40, block=4)
+    a, b = _decoding(sched, [6, 7], max_tokens=9)
     running = sched.schedule()
-    assert not running.items[0].is_final and sched.schedule_ahead(running) is None
+    sched.abort(b.id)
+    assert sched.schedule_ahead(running) is None and not a.awaits_token
 
 
 # ------------------------------------------------------------------ the delay factor, abort, the next batch
