@@ -161,6 +161,7 @@ class HipKernels:
         self.skinny_max_rows = 128
         # up to 8 bfloat16 rows: the product with the norm before it and the residual sum after it folded in
         self.use_rows_gemm = True
+        self.split_library_products = True
         self.rows_waves = 0     # 4 or 8 forces the waves a block of that kernel (0: its own choice)
         self.use_mfma_attention = True
         self.use_tiled_prefill = True
@@ -550,6 +551,19 @@ class HipKernels:
             ctypes.c_float(scale), int(window or 0), self._stream()))
         return out
 
+    def _library_slices(self, m: int, n: int, k: int) -> int:
+        """Into how many slices of K a product that goes to the BLAS library is cut when its reader can add
+        slices.  Measured on an MI355X: with a few hundred rows the library's kernels leave most of the chip idle
+        on products that do not widen (o and down projections: 35 -> 28 us and 96 -> 58 us at 544 rows of the
+        8B shape); with enough rows for 128 tiles of 256 x 256, and for products that widen (whose reader here
+        is the rotation kernel, which wants a tensor for many rows), they are left whole."""
+        if not self.split_library_products or n > k or -(-m // 256) * -(-n // 256) >= 128:
+            return 1
+        for slices in (4, 2):
+            if k % (slices * 8) == 0 and k // slices >= 2048:
+                return slices
+        return 1
+
     def _skinny(self, x, weight) -> bool:
         m, k = x.shape
         return bool(self.use_skinny_gemm and m <= self.skinny_max_rows and x.dtype == torch.bfloat16
@@ -589,6 +603,14 @@ class HipKernels:
             result = DeferredSum(partial, bias, out_dtype)
             return result if defer else self.materialize(result)
         if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and self.allow_library_gemm:
+            slices = self._library_slices(m, n, k) if defer else 1
+            if slices > 1:
+                # a product with too few tiles to fill the chip: K in slices as one batched product with float32
+                # output, left as a sum that the norm behind it adds while it reads
+                part = k // slices
+                partial = torch.bmm(x.view(m, slices, part).transpose(0, 1),
+                                    weight.view(n, slices, part).permute(1, 2, 0), out_dtype=torch.float32)
+                return DeferredSum(partial, bias, out_dtype)
             if bias is None and out_dtype == torch.bfloat16:
                 return torch.nn.functional.linear(x, weight)
             # float32 out, or a bias: the library writes its float32 sums as they are, so that logits have the
