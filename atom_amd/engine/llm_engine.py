@@ -225,6 +225,7 @@ class LLMEngine:
         ahead = None
         if self.deferred_output:
             batch = self.scheduler.schedule_ahead(running.batch)
+            done += self.scheduler.take_rejected()   # requests that the schedule turned away or found aborted
             if batch is not None:
                 ahead = self._launch(batch, {it.seq.id: k for k, it in enumerate(running.finals)})
                 self.steps_launched_ahead += 1

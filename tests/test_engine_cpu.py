@@ -302,3 +302,25 @@ def test_abort_through_the_engine():
     alone = _engine(True).generate([keep.token_ids[:12]], sp)[0]
     assert alone["token_ids"] == keep.completion_token_ids
     _idle(llm)
+
+
+def test_a_request_turned_away_while_steps_run_ahead_still_comes_back():
+    """A request that can never run (longer than max_model_len) arrives while decode steps are launched ahead of
+    each other: it is handed back at once, not when the engine runs dry."""
+    from atom_amd import SamplingParams
+
+    llm = _engine(True, max_model_len=64)
+    sp = SamplingParams(temperature=0.0, max_tokens=25, ignore_eos=True)
+    keep = llm.add_request(random_ids("B", 12, 1), sp)[0]
+    for _ in range(4):
+        llm.step()
+    assert llm.steps_launched_ahead >= 2
+    huge = llm.add_request(random_ids("B", 100, 2), sp)[0]
+    back = []
+    for _ in range(3):
+        back += llm.step()
+    assert [s.id for s in back] == [huge.id] and huge.leave_reason.startswith("unschedulable")
+    while not llm.is_finished():
+        llm.step()
+    assert keep.num_completion_tokens == 25
+    _idle(llm)
