@@ -283,8 +283,7 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
           mx = fmaxf(mx, sc[i]);
         }
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      mx = rows_max(mx);
       const float new_max = fmaxf(run_max[rt], mx * p.scale_log2);
       const float base = new_max == -INFINITY ? 0.f : new_max;
       const float alpha = fast_exp2(run_max[rt] - base);   // 0 while nothing was seen yet
@@ -313,8 +312,7 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     float total = run_sum[rt];
-    total += __shfl_xor(total, 16, kWave);
-    total += __shfl_xor(total, 32, kWave);
+    total = rows_sum(total);
     if (!row_ok[rt]) continue;
     const int row = rt * 16 + r16;
     if (DECODE && p.parts > 1) {
@@ -465,8 +463,7 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave, (D <= 128 ? 2 : 
         for (int e = 0; e < 8; ++e) ss += x[j][e] * x[j][e];
       }
       if (p.q_weight) {
-        ss += __shfl_xor(ss, 16, kWave);
-        ss += __shfl_xor(ss, 32, kWave);
+        ss = rows_sum(ss);
         const float inv = rsqrtf(ss / (float)D + p.eps);
 #pragma unroll
         for (int j = 0; j < KCH; ++j)
@@ -598,8 +595,7 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave, (D <= 128 ? 2 : 
           mx = fmaxf(mx, sc[e]);
         }
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      mx = rows_max(mx);
       const float new_max = fmaxf(run_max[rt], mx * p.scale_log2);
       const float base = new_max == -INFINITY ? 0.f : new_max;
       const float alpha = fast_exp2(run_max[rt] - base);
@@ -632,8 +628,7 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave, (D <= 128 ? 2 : 
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       float total = run_sum[rt];
-      total += __shfl_xor(total, 16, kWave);
-      total += __shfl_xor(total, 32, kWave);
+      total = rows_sum(total);
       const int row = rt * 16 + r16;
 #pragma unroll
       for (int t = 0; t < DT; ++t) *reinterpret_cast<f32x4*>(mine + row * D + 16 * t + 4 * g) = acc[rt][t];
@@ -666,8 +661,7 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave, (D <= 128 ? 2 : 
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     float total = run_sum[rt];
-    total += __shfl_xor(total, 16, kWave);
-    total += __shfl_xor(total, 32, kWave);
+    total = rows_sum(total);
     if (!row_ok[rt]) continue;
     const int row = rt * 16 + r16;
     if (p.parts > 1) {
@@ -806,6 +800,8 @@ static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
 // leaves them in a lane.
 //
 // Needs D % 64 == 0 and page_size % 8 == 0.
+constexpr float kLazyMax = 8.f;
+
 template <int D, int GH, int TK>
 __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_tiled_kernel(AttnParams p) {
   constexpr int KCH = D / 32;
@@ -1004,21 +1000,25 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
             mx = fmaxf(mx, sc[4 * b + i]);
           }
       } else {
-        const int hi = min(row_pos[rt], ke - 1);
-        const int lo = p.window > 0 ? row_pos[rt] - p.window + 1 : 0;
+        // the visible keys, counted from this lane's first key of the tile: 16 b + i is compared with constants
+        const int first = k0 + 4 * g;
+        const int hi = min(row_pos[rt], ke - 1) - first;
+        const int lo = (p.window > 0 ? row_pos[rt] - p.window + 1 : 0) - first;
 #pragma unroll
         for (int b = 0; b < KB; ++b)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int key = k0 + 16 * b + 4 * g + i;
-            const bool vis = key <= hi && key >= lo;
+            const bool vis = 16 * b + i <= hi && 16 * b + i >= lo;
             sc[4 * b + i] = vis ? s[rt][b][i] : -INFINITY;
             mx = fmaxf(mx, sc[4 * b + i]);
           }
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-      const float new_max = fmaxf(run_max[rt], mx * p.scale_log2);
+      mx = rows_max(mx);
+      // The running maximum follows the tile's only when that is larger by more than kLazyMax (in powers of two):
+      // the weights of a tile are then at most 2^kLazyMax instead of 1, which float32 sums and bfloat16 weights hold
+      // as well, and after a row's first tiles nothing has to be scaled again.
+      const float tile_max = mx * p.scale_log2;
+      const float new_max = tile_max > run_max[rt] + kLazyMax ? tile_max : run_max[rt];
       const float base = new_max == -INFINITY ? 0.f : new_max;
       alpha[rt] = fast_exp2(run_max[rt] - base);
       rescale = rescale || alpha[rt] != 1.f;
@@ -1059,8 +1059,7 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     float total = run_sum[rt];
-    total += __shfl_xor(total, 16, kWave);
-    total += __shfl_xor(total, 32, kWave);
+    total = rows_sum(total);
     if (!row_ok[rt]) continue;
     const int row = rt * 16 + r16;
     bf16_t* dst = p.out + ((size_t)(q_begin + my_row0 + row) * p.hq + head) * D;

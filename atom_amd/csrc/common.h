@@ -46,6 +46,26 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// The maximum (the sum) of v over the four lanes r, r + 16, r + 32 and r + 48, in each of them.  The rows of 16
+// lanes change places through the row-swap instructions of gfx950, without a trip through LDS: the first leaves
+// rows (0, 0, 2, 2) of v in one register and rows (1, 1, 3, 3) in the other, the second the lower half of its
+// operand twice in one and the upper half twice in the other.
+__device__ __forceinline__ float rows_max(float v) {
+  const unsigned bits = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+  const unsigned pair = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+  const auto b = __builtin_amdgcn_permlane32_swap(pair, pair, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+__device__ __forceinline__ float rows_sum(float v) {
+  const unsigned bits = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+  const unsigned pair = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+  const auto b = __builtin_amdgcn_permlane32_swap(pair, pair, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // Sum over a block of up to 1024 threads; `scratch` holds one float per wave
 // (16 at most).  Every thread receives the total.  The order of the partial sums
 // is fixed, so the result does not depend on what else runs.

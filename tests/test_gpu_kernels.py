@@ -329,6 +329,31 @@ def test_prefill_tiles_find_a_far_key():
         assert float((got - val).abs().max()) < 0.05 * float(val.abs().max()) + 0.05
 
 
+@pytest.mark.parametrize("per_tile", [3.0, 11.0])
+def test_prefill_scores_that_climb_from_tile_to_tile(per_tile):
+    """Every query's scores rise with the key's position, by `per_tile` powers of two from one tile of 64 keys to
+    the next: below the step at which the tiled kernel moves a row's running maximum (so that the weights of many
+    tiles are taken against an older maximum) and above it (so that it moves with every tile)."""
+    hq, hkv, d, page = 8, 2, 128, 16
+    q_lens, ctx_lens = [400, 1], [1400, 9]
+    q, kc, vc, meta = _attention_case(torch.bfloat16, hq, hkv, d, page, None, q_lens, ctx_lens, seed=21)
+    u = torch.zeros(d)
+    u[5] = 1.0
+    lift = 4.0
+    per_key = per_tile / 64 / 1.4426950408889634 / d ** -0.5 / lift
+    q = (q.float() + lift * u).to(torch.bfloat16)
+    tables = meta("cpu").block_tables
+    kf = kc.float()
+    for key in range(ctx_lens[0]):
+        kf[int(tables[0, key // page]), :, key % page] += per_key * key * u
+    kc = kf.to(torch.bfloat16)
+    out = torch.empty_like(q, device=DEV)
+    gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, None)
+    want = torch.empty_like(q)
+    PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, None)
+    close(out, want, torch.bfloat16)
+
+
 @pytest.mark.parametrize("parts", [1, 2, 7, 64])
 @pytest.mark.parametrize("window", [None, 300])
 def test_decode_split_over_waves(parts, window):
