@@ -105,20 +105,39 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
     for (int rg = 0; rg < 4; ++rg)
       a[4 * slot + rg] = in ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[rg] + kk)) : zero;
   };
+  // The norm's factor of every row, from the partial sums of squares in index order: wave v takes rows v and
+  // v + waves (there are at least four waves and at most eight rows).  The loads of both rows go out together and
+  // ahead of the first quarters of w, so that no wave waits a second time for the cache.
+  float* inv_s = reinterpret_cast<float*>(smem + waves * AREA);    // [8], behind the waves' areas
+  float sq[2][4];
+  if (p.ss) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int m = wave + t * waves;
+      const bool live = m < p.m;
+      const float* parts = p.ss + (size_t)(p.rows ? p.rows[live ? m : 0] : (live ? m : 0)) * p.ss_parts;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = lane + kWave * u;
+        sq[t][u] = (live && i < p.ss_parts) ? parts[i] : 0.f;
+      }
+    }
+  }
 #pragma unroll
   for (int s4 = 0; s4 < 4; ++s4)
     if (s4 < quarters) load_quarter(s4, s4);
-
-  // the norm's factor of every row, from the partial sums of squares in index order: wave v takes rows
-  // v, v + waves, ..; their loads travel behind the first quarters'
-  float* inv_s = reinterpret_cast<float*>(smem + waves * AREA);    // [8], behind the waves' areas
   if (p.ss) {
-    for (int m = wave; m < p.m; m += waves) {
-      const int row = p.rows ? p.rows[m] : m;
-      float sq = 0.f;
-      for (int i = lane; i < p.ss_parts; i += kWave) sq += p.ss[(size_t)row * p.ss_parts + i];
-      sq = wave_sum(sq);
-      if (lane == 0) inv_s[m] = rsqrtf(sq / (float)k + p.eps);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int m = wave + t * waves;
+      if (m >= p.m) continue;
+      float sum = (sq[t][0] + sq[t][1]) + (sq[t][2] + sq[t][3]);
+      if (p.ss_parts > 4 * kWave) {
+        const float* parts = p.ss + (size_t)(p.rows ? p.rows[m] : m) * p.ss_parts;
+        for (int i = lane + 4 * kWave; i < p.ss_parts; i += kWave) sum += parts[i];
+      }
+      sum = wave_sum(sum);
+      if (lane == 0) inv_s[m] = rsqrtf(sum / (float)k + p.eps);
     }
   }
 
