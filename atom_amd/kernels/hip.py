@@ -553,14 +553,20 @@ class HipKernels:
 
     def _library_slices(self, m: int, n: int, k: int) -> int:
         """Into how many slices of K a product that goes to the BLAS library is cut when its reader can add
-        slices.  Measured on an MI355X: with a few hundred rows the library's kernels leave most of the chip idle
-        on products that do not widen (o and down projections: 35 -> 28 us and 96 -> 58 us at 544 rows of the
-        8B shape); with enough rows for 128 tiles of 256 x 256, and for products that widen (whose reader here
-        is the rotation kernel, which wants a tensor for many rows), they are left whole."""
-        if not self.split_library_products or n > k or -(-m // 256) * -(-n // 256) >= 128:
+        slices.  Measured on an MI355X with the o and down products of the 4B, 8B and 32B shapes at 544 to 4,096
+        rows, the add-norm that reads the slices included: the library's kernels leave much of the chip idle
+        while a product has fewer tiles of 256 x 256 than the chip has CUs, and the most slices that keep
+        tiles x slices within the CUs win (8B down: 96 -> 58 us at 544 rows, 140 -> 108 at 1,024, 210 -> 197 at
+        2,048; 32B down 373 -> 247 at 1,024), as long as a slice keeps 2,048 of K, and 4,096 once there are more
+        than 64 tiles.  Products that widen (whose reader here is the rotation kernel, which wants a tensor for
+        many rows) are left whole."""
+        if not self.split_library_products or n > k:
             return 1
+        tiles = -(-m // 256) * -(-n // 256)
         for slices in (4, 2):
-            if k % (slices * 8) == 0 and k // slices >= 2048:
+            per = k // slices
+            if (k % (slices * 8) == 0 and tiles * slices <= self.num_cus and per >= 2048
+                    and (tiles <= 64 or per >= 4096)):
                 return slices
         return 1
 
