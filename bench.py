@@ -219,6 +219,8 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
                     help="the mixed workload with N requests on the chosen shape (what --shape 4b runs with 32)")
+    ap.add_argument("--budget", type=int, default=None,
+                    help="the scheduler's token budget of a step (mixed: 512 + N by default, so that portions stay 512)")
     ap.add_argument("--temperature", type=float, default=0.0, help="of the decode steps' sampling (0: greedy)")
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--top-k", type=int, default=-1)
@@ -255,6 +257,7 @@ def main() -> int:
         max_seqs = max(points + [mixed])
         max_model_len = args.max_model_len or max(4096, 2 * args.context)
         pages, budget = max_seqs * max_model_len // block, (512 + mixed if mixed else 16384)
+    budget = args.budget or budget
     t0 = time.time()
     llm = LLMEngine(f"{name.lower()}-random", model_config=cfg, load_dummy="random", seed=seed, dtype="bf16",
                     max_model_len=max_model_len, kv_cache_block_size=block, num_kvcache_blocks=pages,

@@ -402,6 +402,26 @@ def test_far_key_among_hundreds(dtype):
             close(out, want, dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_far_key_in_a_long_context(dtype):
+    """Contexts of 70,000 and 65,000 keys (over 4,000 pages a request, scattered over the pool): one key near the
+    start carries the weight for the last row of a prompt portion and for a decode row."""
+    hq, hkv, d, page = 8, 2, 128, 16
+    for b, key in ((0, 1234), (1, 40001)):
+        q, kc, vc, meta = _attention_case(dtype, hq, hkv, d, page, None, [64, 1], [70000, 65000], seed=b,
+                                          scale_one=(b, key, 3.0))
+        out = torch.empty_like(q, device=DEV)
+        gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, None)
+        want = torch.empty_like(q)
+        PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, None)
+        close(out, want, dtype)
+        row = 63 if b == 0 else 64
+        m = meta("cpu")
+        pg, off = int(m.block_tables[b, key // page]), key % page
+        got, val = out[row, hq - 1].float().cpu(), vc[pg, hkv - 1, :, off].float()
+        assert float((got - val).abs().max()) < 0.05 * float(val.abs().max()) + 0.05
+
+
 def test_window_edge():
     """Keys exactly at the window's edge: position p - W + 1 is seen, p - W is not."""
     w = 40
