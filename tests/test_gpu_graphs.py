@@ -11,7 +11,7 @@ from atom_amd.engine.core import StepEntry
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [40, 17, 90, 128], "B": [1, 9, 71, 200, 130], "C": [50, 600, 95, 257], "D": [45, 500, 130, 260]}
+LENGTHS = {"A": [40, 17, 90, 128], "B": [1, 9, 71, 200, 130], "C": [50, 600, 95, 257], "D": [45, 500, 130, 260], "E": [33, 150, 64, 210]}
 
 
 def _requests(which):
@@ -19,7 +19,7 @@ def _requests(which):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("cut", ["tail", "mixed"])
 def test_graph_cuts_match_plain(which, cut, dtype):
     requests = _requests(which)

@@ -13,7 +13,7 @@ from tiny import CONFIGS
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [5, 17, 33, 100, 128, 64], "B": [1, 9, 40, 71, 200, 256, 130], "C": [3, 50, 600, 320, 95, 31, 257, 1000],
-           "D": [2, 70, 700, 129, 33, 400]}
+           "D": [2, 70, 700, 129, 33, 400], "E": [4, 37, 150, 64, 210]}
 
 
 def _requests(which, seed=0):
@@ -32,7 +32,7 @@ def _oracle(which, requests):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
 def test_cuts_match_plain(which, cut, dtype):
     requests = _requests(which)
