@@ -46,6 +46,7 @@ class EngineArgs:
     max_num_seqs: int = 512
     gpu_memory_utilization: float = 0.9
     cudagraph_capture_sizes: str = "[1,2,4,8,16,32,48,64,128,256]"
+    cudagraph_prefill_sizes: str = "[]"
     load_dummy: str | None = None
     torch_profiler_dir: str | None = None
     mark_trace: bool = False
@@ -77,6 +78,9 @@ class EngineArgs:
         parser.add_argument("--gpu-memory-utilization", type=float, default=0.9, help="Share of GPU memory to use.")
         parser.add_argument("--cudagraph-capture-sizes", type=str, default="[1,2,4,8,16,32,48,64,128,256]",
                             help="Decode batch sizes captured as HIP graphs.")
+        parser.add_argument("--cudagraph-prefill-sizes", type=str, default="[]",
+                            help="Ours: prompt-token capacities of graphs for steps with prompt portions beside decode "
+                                 "tokens, e.g. [512]; empty (the default): such steps are launched one by one, ahead of time.")
         parser.add_argument("--load-dummy", type=str, nargs="?", const="random", default=None,
                             help="Skip the checkpoint: seeded random weights.")
         parser.add_argument("--torch-profiler-dir", type=str, default=None, help="Write a torch.profiler trace here.")
@@ -107,6 +111,7 @@ class EngineArgs:
         kwargs = {f.name: getattr(self, f.name) for f in fields(self) if f.name != "model"}
         kwargs["kv_cache_block_size"] = kwargs.pop("block_size")
         kwargs["cudagraph_capture_sizes"] = parse_size_list(kwargs["cudagraph_capture_sizes"])
+        kwargs["cudagraph_prefill_sizes"] = parse_size_list(kwargs["cudagraph_prefill_sizes"])
         kwargs.pop("level")
         if kwargs.pop("cudagraph_mode") == "NONE":
             kwargs["enforce_eager"] = True

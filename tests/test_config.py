@@ -121,3 +121,11 @@ def test_cli_flags_in_both_spellings():
     kw = a._get_engine_kwargs()
     assert kw["kv_cache_block_size"] == 32 and "block_size" not in kw
     assert kw["cudagraph_capture_sizes"][:3] == [1, 2, 4]
+
+
+def test_cli_graph_sizes_for_steps_with_prompt_portions():
+    parser = FlexibleArgumentParser()
+    EngineArgs.add_cli_args(parser)
+    off = EngineArgs.from_cli_args(parser.parse_args(["--model", "m"]))._get_engine_kwargs()
+    on = EngineArgs.from_cli_args(parser.parse_args(["--model", "m", "--cudagraph-prefill-sizes", "[256, 512]"]))
+    assert off["cudagraph_prefill_sizes"] == [] and on._get_engine_kwargs()["cudagraph_prefill_sizes"] == [256, 512]
