@@ -115,6 +115,7 @@ class PendingProduct:
 
     def __init__(self, x, weight, bias, dtype: torch.dtype):
         self.x, self.weight, self.bias, self.dtype = x, weight, bias, dtype
+        self.split = False   # set by a norm that wants the product as a sum of K slices (see pending_norm)
 
     @property
     def shape(self):
@@ -298,6 +299,19 @@ class HipKernels:
                     and (isinstance(x, PendingNorm) or x.dtype == torch.bfloat16)
                     and self.lib.atom_gemm_rows_supports(m, weight.shape[0], k))
 
+    def _rows_residual_pays(self, n: int, k: int) -> bool:
+        """Whether the few-rows product with the residual sum folded in beats the product with K cut between
+        blocks followed by the add-norm kernel.  The folded one owns 16 columns and all of K per block, so its
+        n / 16 blocks are all the parallelism there is, and it takes as long as its busiest CU needs for its
+        blocks' rows of w.  Measured on an MI355X at 8 rows: a CU draws 28 GB/s at most (22 when all 256 share the
+        chip's 5.6 TB/s), a kernel costs 3.4 us beside that and the add-norm kernel 5 us.  32B down (320 blocks, 2 on
+        64 of the CUs): 61.7 us against 48.4 + 5.2 the split way; 32B o: 22.7 against 19.3 + 5.2; 4B down (160
+        blocks): 14.6 against 11.2 + 4.7; 8B down (256 blocks): 21.2 against 19.5 + 4.7."""
+        tiles = -(-n // 16)
+        folded = max(tiles * 32 * k / 5.6e6, -(-tiles // self.num_cus) * 32 * k / 28e3)   # the chip's pace, the busiest CU's
+        split = n * k * 2 / 5.5e6 + 5.0
+        return folded <= split
+
     def _rows_launch(self, x, weight, bias, mode: int, y=None, res=None, ss_out=None, xg_out=None, g_next=None,
                      out_f32: bool = False):
         m, k = x.shape
@@ -330,6 +344,9 @@ class HipKernels:
         if not isinstance(x, PendingProduct) or residual is None:
             return None
         m, n = x.shape
+        if not self._rows_residual_pays(n, x.weight.shape[1]) and not isinstance(x.x, PendingNorm):
+            x.split = True    # rmsnorm() launches it with K cut between blocks and adds the slices itself
+            return None
         self._check("residual", residual, torch.float32, (m, n))
         self._check("norm weight", weight, torch.float32, (n,))
         inner = x.x
@@ -368,6 +385,8 @@ class HipKernels:
         """mode 'plain': out = norm(x); 'init': residual = x, out = norm(x);
         'add': residual += x, out = norm(residual).  With ``rows`` only those source
         rows are normed (into out[0..len(rows))) and the residual is not written."""
+        if isinstance(x, PendingProduct) and x.split:
+            x = self.linear(x.x, x.weight, x.bias, x.dtype, defer=True, few_rows=False)
         if isinstance(x, (PendingProduct, PendingNorm)):
             x = self.materialize(x)
         width = x.shape[-1]
@@ -575,7 +594,7 @@ class HipKernels:
         return bool(self.use_skinny_gemm and m <= self.skinny_max_rows and x.dtype == torch.bfloat16
                     and weight.dtype == torch.bfloat16 and self.lib.atom_gemm_skinny_supports(m, weight.shape[0], k))
 
-    def linear(self, x, weight, bias=None, out_dtype=None, defer: bool = False):
+    def linear(self, x, weight, bias=None, out_dtype=None, defer: bool = False, few_rows: bool = True):
         """``x @ weight.T (+ bias)``.  bfloat16 operands with at most 64 rows (narrow products: 128) run this
         library's own weight-streaming kernels; with more rows they go to the BLAS library, as the reference's engine
         does for its matrix products; anything with a float32 operand runs this library's float32
@@ -585,7 +604,7 @@ class HipKernels:
             x = self.materialize(x)
         m, k = x.shape
         n = weight.shape[0]
-        if m and self._rows_takes(x, weight):
+        if m and few_rows and self._rows_takes(x, weight):
             if defer:
                 return PendingProduct(x, weight, bias, out_dtype or x.dtype)
             return self._rows_product(x, weight, bias, out_dtype or x.dtype)

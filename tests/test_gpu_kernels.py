@@ -728,6 +728,7 @@ def test_rows_product_plain_gate_and_residual(m, n, k, waves):
 
     ops = gpu_ops()
     ops.rows_waves = waves
+    ops._rows_residual_pays = lambda n, k: True   # the folded residual sum at every size, also where the split way is faster
     try:
         x = rnd((m, k), torch.bfloat16, 50, 1.0)
         w = rnd((n, k), torch.bfloat16, 51, 0.05)
@@ -780,6 +781,34 @@ def test_rows_product_plain_gate_and_residual(m, n, k, waves):
                 assert torch.equal(y3[0], y2[m - 1]) and torch.equal(y3[1], y2[0])
     finally:
         ops.rows_waves = 0
+        del ops._rows_residual_pays
+
+
+def test_residual_product_with_too_few_tiles_goes_the_split_way():
+    """A product of 160 column tiles and a long K (135 MB of weights): the few-rows kernel with the residual sum
+    folded in would leave 96 CUs idle, so the norm launches the product with K cut between blocks and adds the
+    slices itself; the same numbers come out."""
+    from atom_amd.kernels.hip import DeferredSum, PendingProduct
+
+    ops = gpu_ops()
+    m, n, k = 5, 2560, 26400
+    assert not ops._rows_residual_pays(n, k) and not ops._rows_residual_pays(5120, 25600)
+    assert all(ops._rows_residual_pays(*nk) for nk in [(4096, 12288), (4096, 4096), (2560, 9728), (2560, 4096), (5120, 8192)])
+    x = rnd((m, k), torch.bfloat16, 70, 1.0)
+    w = rnd((n, k), torch.bfloat16, 71, 0.02)
+    want = x.double() @ w.double().T
+    res = rnd((m, n), torch.float32, 72, 2.0)
+    gamma = 1 + rnd((n,), torch.float32, 73, 0.2)
+    pending = ops.linear(x.to(DEV), w.to(DEV), None, defer=True)
+    assert isinstance(pending, PendingProduct)
+    res_gpu = res.to(DEV)
+    assert ops.pending_norm(pending, res_gpu, gamma.to(DEV), 1e-6) is None and pending.split
+    assert isinstance(ops.linear(x.to(DEV), w.to(DEV), None, defer=True, few_rows=False), DeferredSum)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    ops.rmsnorm(pending, gamma.to(DEV), 1e-6, out, residual=res_gpu, mode="add")
+    new_res = res.double() + want
+    assert float((res_gpu.cpu().double() - new_res).abs().max()) <= 1e-4 * float(new_res.abs().max())
+    close(out, new_res * torch.rsqrt(new_res.pow(2).mean(-1, keepdim=True) + 1e-6) * gamma.double(), torch.bfloat16)
 
 
 def test_rows_product_gate_alone_and_odd_widths():
