@@ -149,6 +149,46 @@ def run_mixed(llm, args, name, raw, layers, gen, requests: int) -> dict:
     }
 
 
+def run_single(llm, args, name, raw, layers, gen, pairs) -> dict:
+    """One request at a time: time to the first token, time per output token and output tokens a second as
+    the reference prints them for its single-stream runs (atom/model_engine/llm_engine.py:735-744: TTFT =
+    first token - arrival, TPOT = (leave - first token) / (output tokens - 1)), for its own input / output lengths
+    (recipes/Qwen3-8B-FP8.md:69-73: 18 / 80 and 549 / 256)."""
+    import torch
+    from atom_amd import SamplingParams
+
+    vocab = raw["vocab_size"]
+    llm.generate([torch.randint(0, vocab, (64,), generator=gen).tolist()],
+                 SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))   # untimed: first-use work
+    rows = {}
+    for isl, osl in pairs:
+        best = None
+        for _ in range(3):
+            p = torch.randint(0, vocab, (isl,), generator=gen).tolist()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            out = llm.generate([p], SamplingParams(temperature=0.0, max_tokens=osl, ignore_eos=True))[0]
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - t
+            if best is None or wall < best[0]:
+                best = (wall, out)
+        wall, out = best
+        rows[f"isl{isl}_osl{osl}"] = {"ttft_ms": round(out["ttft"] * 1e3, 2), "tpot_ms": round(out["tpot"] * 1e3, 3),
+                                      "output_tok_s": round(osl / wall, 1)}
+        print(f"[bench] single stream, {isl} in / {osl} out: {rows[f'isl{isl}_osl{osl}']}", file=sys.stderr, flush=True)
+    isl, osl = pairs[-1]
+    last = rows[f"isl{isl}_osl{osl}"]
+    return {
+        "metric": f"single-stream output tok/s, {isl} tokens in / {osl} out ({name}, bf16)",
+        "value": last["output_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": osl, "warmup": 0,
+        "ms_per_step": last["tpot_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic: seeded uniform random token ids, seeded random N(0, 0.02) weights",
+        "config": flat_config(name, raw, layers, global_batch=1, seq_len=isl + osl, hip_graphs=not args.enforce_eager,
+                              deferred_output=not args.no_deferred_output),
+        "single_stream": rows,
+    }
+
+
 def run_long(llm, args, name, raw, layers, gen, batch: int = 16, prompt_len: int = 8192, out_tokens: int = 256) -> dict:
     """Long prompts prefilled in portions of the token budget, then the whole batch decodes."""
     import torch
@@ -219,6 +259,8 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
                     help="the mixed workload with N requests on the chosen shape (what --shape 4b runs with 32)")
+    ap.add_argument("--single", type=str, default="", metavar="ISL,OSL[;ISL,OSL]",
+                    help="one request at a time: TTFT, TPOT and output tok/s, e.g. '18,80;549,256' (the reference's own pairs)")
     ap.add_argument("--budget", type=int, default=None,
                     help="the scheduler's token budget of a step (mixed: 512 + N by default, so that portions stay 512)")
     ap.add_argument("--temperature", type=float, default=0.0, help="of the decode steps' sampling (0: greedy)")
@@ -247,8 +289,8 @@ def main() -> int:
     layers = args.layers or full_layers
     raw["num_hidden_layers"] = layers
     cfg = model_config_from_dict(raw)
-    mixed = args.mixed or (32 if args.shape == "4b" else 0)
-    long_run = args.shape == "32b" and not mixed
+    mixed = 0 if args.single else (args.mixed or (32 if args.shape == "4b" else 0))
+    long_run = args.shape == "32b" and not mixed and not args.single
     points = sorted({int(x) for x in args.points.split(",") if x} | {args.batch})
     block = 16
     if long_run:
@@ -275,6 +317,10 @@ def main() -> int:
     def sync():
         torch.cuda.synchronize()
 
+    if args.single:
+        pairs = [tuple(int(v) for v in pair.split(",")) for pair in args.single.split(";")]
+        print(json.dumps(run_single(llm, args, name, raw, layers, gen, pairs)), flush=True)
+        return 0
     if mixed:
         print(json.dumps(run_mixed(llm, args, name, raw, layers, gen, mixed)), flush=True)
         return 0
