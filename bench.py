@@ -259,6 +259,8 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
                     help="the mixed workload with N requests on the chosen shape (what --shape 4b runs with 32)")
+    ap.add_argument("--decode", action="store_true",
+                    help="the prefill and decode points (what --shape 8b runs) on the chosen shape, whatever its own workload")
     ap.add_argument("--single", type=str, default="", metavar="ISL,OSL[;ISL,OSL]",
                     help="one request at a time: TTFT, TPOT and output tok/s, e.g. '18,80;549,256' (the reference's own pairs)")
     ap.add_argument("--budget", type=int, default=None,
@@ -289,8 +291,9 @@ def main() -> int:
     layers = args.layers or full_layers
     raw["num_hidden_layers"] = layers
     cfg = model_config_from_dict(raw)
-    mixed = 0 if args.single else (args.mixed or (32 if args.shape == "4b" else 0))
-    long_run = args.shape == "32b" and not mixed and not args.single
+    plain = bool(args.single) or args.decode
+    mixed = 0 if plain else (args.mixed or (32 if args.shape == "4b" else 0))
+    long_run = args.shape == "32b" and not mixed and not plain
     points = sorted({int(x) for x in args.points.split(",") if x} | {args.batch})
     block = 16
     if long_run:
