@@ -5,6 +5,7 @@ architecture; an architecture is a function from its configuration to a ``ModelS
 
 from __future__ import annotations
 
+import re
 from dataclasses import dataclass
 
 import torch
@@ -37,6 +38,11 @@ class ModelSpec:
     final_norm_prefix: str = "model.norm"
     head_prefix: str = "lm_head"
     ignorable: tuple[str, ...] = ()          # checkpoint tensors that may be present and are not used
+    # checkpoint tensors dropped by the form of their name (atom/model_loader/weight_names.py:160-188): cache
+    # scales, rotation tables that a checkpoint still carries, whatever starts with a prefix the model names
+    drop_suffixes: tuple[str, ...] = ("kv_scale",)
+    drop_substrings: tuple[str, ...] = ("inv_freq",)
+    drop_prefixes: tuple[str, ...] = ()
 
     def running_order(self) -> list[LayerRun]:
         return list(self.order) if self.order is not None else [LayerRun(i) for i in range(len(self.blocks))]
@@ -67,11 +73,33 @@ class CausalLM(Part):
         self.ignorable = set(spec.ignorable)
         if spec.tie_word_embeddings:
             self.ignorable.add(f"{spec.head_prefix}.weight")
+        head, _, tail = spec.layer_prefix.partition("{}")
+        self._layer_name = re.compile(re.escape(head) + r"(\d+)" + (re.escape(tail) if tail else "") + r"\.")
         self.dtype: torch.dtype | None = None
         self.device: torch.device | None = None
 
     def children(self):
         return [self.embedding, *self.blocks, self.final_norm, self.head]
+
+    def drops(self, name: str) -> str | None:
+        """Why a checkpoint tensor that no parameter names is left aside without an error, or None if it
+        is not: the exact names of ``ignorable``, the name forms of the reference's checkpoint rewriter
+        (atom/model_loader/weight_names.py:160-188: ``*kv_scale``, ``*inv_freq*``, model-declared
+        prefixes) and the tensors of layers beyond the model's last (``_is_past_last_layer``, :197-201:
+        a checkpoint run with fewer layers than it holds)."""
+        spec = self.spec
+        if name in self.ignorable:
+            return "not used by this model"
+        if any(name.endswith(s) for s in spec.drop_suffixes):
+            return "a cache scale"
+        if any(s in name for s in spec.drop_substrings):
+            return "a table the engine computes itself"
+        if any(name.startswith(p) for p in spec.drop_prefixes):
+            return "under a prefix the model leaves out"
+        match = self._layer_name.search(name)
+        if match is not None and int(match.group(1)) >= len(self.blocks):
+            return f"of a layer beyond the model's {len(self.blocks)}"
+        return None
 
     @property
     def vocab_size(self) -> int:

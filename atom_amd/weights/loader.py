@@ -8,18 +8,25 @@ kept in bfloat16 for serving (a matrix the checkpoint stores in 32-bit stays 32-
 or widened to float32 on the 32-bit path; norm weights and biases are float32; integer
 tensors become int32.  Unlike the reference, which only warns
 (atom/model_loader/loading_core.py:389-468), anything missing, unexpected or
-mis-shaped is one error that lists all of it.
+mis-shaped is one error that lists all of it.  What the reference's checkpoint rewriter
+drops by the form of a name (atom/model_loader/weight_names.py:160-201: cache scales,
+``inv_freq`` tables, layers beyond ``num_hidden_layers``) is dropped here too, through
+the model's ``drops(name)``, with a debug line in the log.
 """
 
 from __future__ import annotations
 
 import json
+import logging
 import os
 from typing import Callable
 
 import torch
 
 from ..parts.base import ParamSpec, Part
+
+
+logger = logging.getLogger("atom_amd")
 
 
 class WeightError(RuntimeError):
@@ -149,9 +156,17 @@ def load_weights(model: Part, source: TensorSource, device, dtype: torch.dtype,
     """Fills every declared parameter of ``model`` from ``source`` or raises ``WeightError``."""
     expected = expected_tensors(model)
     present = set(source.names())
-    ignorable = getattr(model, "ignorable", set())
+    drops = getattr(model, "drops", None)
     missing = [n for n in expected if n not in present]
-    unexpected = [n for n in present if n not in expected and n not in ignorable]
+    unexpected = []
+    for n in sorted(present):
+        if n in expected:
+            continue
+        why = drops(n) if drops is not None else None
+        if why is None:
+            unexpected.append(n)
+        else:
+            logger.debug("checkpoint tensor %s dropped: %s", n, why)
     mismatched = [(n, source.shape(n), shape) for n, (shape, _) in expected.items()
                   if n in present and tuple(source.shape(n)) != tuple(shape)]
     if missing or unexpected or mismatched:

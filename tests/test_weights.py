@@ -87,19 +87,64 @@ def test_one_error_lists_missing_unexpected_and_misshaped():
     state = random_state_dict(cfg, 1)
     del state["model.layers.0.mlp.up_proj.weight"]
     del state["model.norm.weight"]
-    state["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)
+    state["model.layers.0.self_attn.gate.weight"] = torch.zeros(16)
     state["model.layers.2.self_attn.o_proj.weight"] = torch.zeros(192, 96)     # transposed
     state["model.layers.1.self_attn.k_norm.weight"] = torch.zeros(31)
     with pytest.raises(WeightError) as e:
         load_weights(build_model(cfg), DictSource(state, "test"), "cpu", torch.bfloat16)
     err = e.value
     assert err.missing == ["model.layers.0.mlp.up_proj.weight", "model.norm.weight"]
-    assert err.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert err.unexpected == ["model.layers.0.self_attn.gate.weight"]
     assert [m[0] for m in err.mismatched] == ["model.layers.1.self_attn.k_norm.weight",
                                               "model.layers.2.self_attn.o_proj.weight"]
     text = str(err)
     for needle in ("missing (2)", "unexpected (1)", "wrong shape (2)", "(192, 96)", "(96, 192)", "up_proj"):
         assert needle in text
+
+
+def test_names_the_reference_drops_are_dropped(caplog):
+    """atom/model_loader/weight_names.py:160-201: ``*kv_scale``, ``*inv_freq*`` and layers beyond the
+    model's last are left aside without an error; a name that only looks similar is still an error."""
+    import logging
+    cfg = model_config_from_dict(TINY_B)
+    state = random_state_dict(cfg, 1)
+    state["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)
+    state["model.layers.1.self_attn.k_proj.kv_scale"] = torch.ones(1)
+    state[f"model.layers.{cfg.num_hidden_layers}.mlp.up_proj.weight"] = torch.zeros(3, 3)
+    state[f"model.layers.{cfg.num_hidden_layers + 7}.anything"] = torch.zeros(2)
+    with caplog.at_level(logging.DEBUG, logger="atom_amd"):
+        model = build_model(cfg)
+        load_weights(model, DictSource(state), "cpu", torch.bfloat16)
+    dropped = [r.getMessage() for r in caplog.records if "dropped" in r.getMessage()]
+    assert len(dropped) == 4 and any("inv_freq" in d for d in dropped)
+    state["model.layers.0.self_attn.kv_scales"] = torch.ones(1)      # neither suffix nor substring
+    state["model.layers.x.mlp.up_proj.weight"] = torch.ones(1)       # no layer number
+    with pytest.raises(WeightError) as e:
+        load_weights(build_model(cfg), DictSource(state), "cpu", torch.bfloat16)
+    assert e.value.unexpected == ["model.layers.0.self_attn.kv_scales", "model.layers.x.mlp.up_proj.weight"]
+    assert not e.value.missing and not e.value.mismatched
+
+
+def test_a_checkpoint_runs_with_fewer_layers_than_it_holds(tmp_path):
+    """The reference's truncation path: ``--hf-overrides '{"num_hidden_layers": N}'`` (atom/config.py:1699-1701)
+    with the tensors of the layers past N dropped by name (weight_names.py:197-201)."""
+    from atom_amd.config import Config
+    folder = tiny_folder("B")                      # three layers
+    full = Config(model=folder, dtype="fp32")
+    cut = Config(model=folder, dtype="fp32", hf_overrides={"num_hidden_layers": 2})
+    assert full.model_config.num_hidden_layers == 3 and cut.model_config.num_hidden_layers == 2
+    small, whole = build_model(cut.model_config), build_model(full.model_config)
+    load_model_folder(small, folder, "cpu", torch.float32)
+    load_model_folder(whole, folder, "cpu", torch.float32)
+    assert len(small.blocks) == 2
+    for a, b in zip(small.blocks, whole.blocks):
+        for pa, pb in zip(a.walk(), b.walk()):
+            for name in pa.params:
+                assert torch.equal(pa.params[name], pb.params[name])
+    # more layers than the checkpoint holds is still an error that names what is missing
+    more = Config(model=folder, dtype="fp32", hf_overrides={"num_hidden_layers": 4})
+    with pytest.raises(WeightError, match=r"model\.layers\.3\."):
+        load_model_folder(build_model(more.model_config), folder, "cpu", torch.float32)
 
 
 def test_untied_model_needs_its_head():
