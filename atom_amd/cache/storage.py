@@ -57,10 +57,16 @@ def plan_cache(model, page_size: int, dtype: torch.dtype, *, num_pages: int | No
     for run, group in zip(model.order, run_group):
         if run.reads_run is not None:
             continue
-        need = model.blocks[run.layer].mixer.cache_need()
+        mixer = model.blocks[run.layer].mixer
+        need = mixer.cache_need()
         kind = kind_of(need)
         if kind is None:
             continue
+        if group is not None:
+            problem = mixer.page_size_problem(page_size)
+            if problem:
+                raise ValueError(f"cache pages of {page_size} tokens do not suit layer {run.layer} "
+                                 f"({type(mixer).__name__}): {problem}")
         per_slot += kind.request_bytes(need, dtype)
         if group is not None:
             per_page[group] += kind.page_bytes(need, page_size, dtype)

@@ -35,6 +35,7 @@ class Config:
     # Off by default: on an MI355X such steps keep the GPU busy when launched one by one, as long as they are
     # launched ahead (deferred_output), and a graph pads every step to its bucket.
     cudagraph_prefill_sizes: list[int] = field(default_factory=list)
+    cudagraph_prefill_slots: int = 2      # prompt portions such a graph holds at most
     hf_overrides: dict | None = None
     dtype: str = "bf16"
     seed: int = 0
@@ -62,8 +63,8 @@ class Config:
         if self.max_model_len is None:
             self.max_model_len = mc.max_position_embeddings
         self.max_model_len = min(self.max_model_len, mc.max_position_embeddings)
-        if self.kv_cache_block_size <= 0 or self.kv_cache_block_size % 4:
-            raise ConfigError("kv_cache_block_size must be a positive multiple of 4")
+        if self.kv_cache_block_size <= 0:     # what else a page size must be is the mixers' to say (plan_cache)
+            raise ConfigError("kv_cache_block_size must be positive")
         # atom/config.py:1755-1767
         if self.long_prefill_token_threshold:
             if self.long_prefill_token_threshold > self.max_model_len:

@@ -47,6 +47,7 @@ class EngineArgs:
     gpu_memory_utilization: float = 0.9
     cudagraph_capture_sizes: str = "[1,2,4,8,16,32,48,64,128,256]"
     cudagraph_prefill_sizes: str = "[]"
+    cudagraph_prefill_slots: int = 2
     load_dummy: str | None = None
     torch_profiler_dir: str | None = None
     mark_trace: bool = False
@@ -81,6 +82,8 @@ class EngineArgs:
         parser.add_argument("--cudagraph-prefill-sizes", type=str, default="[]",
                             help="Ours: prompt-token capacities of graphs for steps with prompt portions beside decode "
                                  "tokens, e.g. [512]; empty (the default): such steps are launched one by one, ahead of time.")
+        parser.add_argument("--cudagraph-prefill-slots", type=int, default=2,
+                            help="Ours: prompt portions one such graph holds at most.")
         parser.add_argument("--load-dummy", type=str, nargs="?", const="random", default=None,
                             help="Skip the checkpoint: seeded random weights.")
         parser.add_argument("--torch-profiler-dir", type=str, default=None, help="Write a torch.profiler trace here.")

@@ -43,7 +43,7 @@ class StepEntry:
 class EngineCore:
     def __init__(self, model, ops, plan: CachePlan, max_num_seqs: int, device, dtype: torch.dtype,
                  graph_sizes: list[int] | None = None, max_model_len: int = 0, prefix_caching: bool = False,
-                 graph_prefill_sizes: list[int] | None = None):
+                 graph_prefill_sizes: list[int] | None = None, graph_prefill_slots: int | None = None):
         self.model = model
         self.ops = ops
         self.device = torch.device(device)
@@ -74,7 +74,8 @@ class EngineCore:
         if graph_sizes:
             from .graphs import DecodeGraphs
 
-            graphs = DecodeGraphs(self, graph_sizes, max_model_len or self.max_positions, graph_prefill_sizes)
+            graphs = DecodeGraphs(self, graph_sizes, max_model_len or self.max_positions, graph_prefill_sizes,
+                                  **({} if graph_prefill_slots is None else {"prefill_slots": graph_prefill_slots}))
             self.graphs = graphs if graphs.usable else None
 
     # ------------------------------------------------------------------ requests
@@ -325,7 +326,8 @@ def load_model(model_dir: str | None, *, dtype: torch.dtype, device, model_confi
 def build_core(model, ops, *, dtype: torch.dtype, device, page_size: int = 16, num_pages: int | None = None,
                budget_bytes: int | None = None, max_num_seqs: int = 4, max_model_len: int = 0,
                max_num_batched_tokens: int = 0, graph_sizes: list[int] | None = None,
-               prefix_caching: bool = False, graph_prefill_sizes: list[int] | None = None) -> EngineCore:
+               prefix_caching: bool = False, graph_prefill_sizes: list[int] | None = None,
+               graph_prefill_slots: int | None = None) -> EngineCore:
     from ..cache.storage import plan_cache
 
     plan = plan_cache(model, page_size, dtype, num_pages=num_pages, budget_bytes=budget_bytes,
@@ -333,4 +335,4 @@ def build_core(model, ops, *, dtype: torch.dtype, device, page_size: int = 16, n
                       max_num_batched_tokens=max_num_batched_tokens)
     return EngineCore(model, ops, plan, max_num_seqs, device, dtype, graph_sizes=graph_sizes,
                       max_model_len=max_model_len, prefix_caching=prefix_caching,
-                      graph_prefill_sizes=graph_prefill_sizes)
+                      graph_prefill_sizes=graph_prefill_sizes, graph_prefill_slots=graph_prefill_slots)

@@ -37,6 +37,9 @@ import torch
 from .context import StepContext
 
 
+PREFILL_SLOTS = 2    # prompt portions a replayed step holds at most, unless the engine's configuration says otherwise
+
+
 class _Captured:
     def __init__(self, shape: tuple[int, int, int]):
         self.shape = shape                      # (P prompt-token rows, R portion slots, N single-token rows)
@@ -59,7 +62,7 @@ class _Captured:
 
 class DecodeGraphs:
     def __init__(self, core, sizes: list[int], max_model_len: int, prefill_sizes: list[int] | None = None,
-                 prefill_slots: int = 2):
+                 prefill_slots: int = PREFILL_SLOTS):
         self.core = core
         limit = core.manager.slots.num_slots
         self.sizes = sorted({int(s) for s in sizes if 0 < int(s) <= limit})
@@ -246,8 +249,8 @@ class DecodeGraphs:
                           cu_seqlens_q=view("starts"), context_lens=view("context_lens"),
                           cached_lens=view("cached_lens"), slot_of_seq=view("slot_of_seq"),
                           num_prefill=cap.first_single, max_q_len=max(p, 1),
-                          max_context_len=max(w * g.page_size for w, g in zip(self.widths, core.manager.groups))
-                          if self.widths else self.max_model_len, replayed=True)
+                          # a bound, not the batch's own: no request of a replayed step is longer (accepts())
+                          max_context_len=self.max_model_len, replayed=True)
         for gi, (g, width) in enumerate(zip(core.manager.groups, self.widths)):
             ctx.block_tables[gi] = view(f"bt{gi}").view(cap.num_seqs, width)
             ctx.slot_mappings[gi] = view(f"slots{gi}")

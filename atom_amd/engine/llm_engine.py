@@ -101,7 +101,8 @@ class LLMEngine:
             max_num_seqs=cfg.max_num_seqs, max_model_len=cfg.max_model_len,
             max_num_batched_tokens=cfg.max_num_batched_tokens,
             graph_sizes=None if cfg.enforce_eager else cfg.cudagraph_capture_sizes,
-            graph_prefill_sizes=cfg.cudagraph_prefill_sizes, prefix_caching=cfg.enable_prefix_caching)
+            graph_prefill_sizes=cfg.cudagraph_prefill_sizes, graph_prefill_slots=cfg.cudagraph_prefill_slots,
+            prefix_caching=cfg.enable_prefix_caching)
         self._log_capacity()
         if self.core.graphs is not None:   # as the reference's engine does before it serves (engine_core.py:131-138)
             captured = self.core.graphs.capture_all()
@@ -145,8 +146,15 @@ class LLMEngine:
             return 0
         widest = max((int(p.shape[0]) for block in self.model.blocks for part in block.walk()
                       for p in part.params.values() if p.dim() == 2), default=spec.hidden_size)
-        live = max(sizes) * (4 * spec.hidden_size + 8 * widest) * 4
-        return sum(sizes) * spec.vocab_size * 4 + 2 * live + (128 << 20)
+        rows, logits_rows = max(sizes), sum(sizes)
+        if cfg.cudagraph_prefill_sizes:
+            # a graph per (portion tokens P, single tokens N >= 8): logits at the portion slots and the single
+            # tokens, activations for P + N rows
+            mixed = [s for s in sizes if s >= 8] or sizes[-1:]
+            logits_rows += len(cfg.cudagraph_prefill_sizes) * sum(cfg.cudagraph_prefill_slots + n for n in mixed)
+            rows = max(rows, max(cfg.cudagraph_prefill_sizes) + max(mixed))
+        live = rows * (4 * spec.hidden_size + 8 * widest) * 4
+        return logits_rows * spec.vocab_size * 4 + 2 * live + (128 << 20)
 
     def _log_capacity(self) -> None:
         """How many requests the pages hold at once, by context length

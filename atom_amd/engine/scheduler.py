@@ -346,7 +346,13 @@ class Scheduler:
         the pages of one more token for every decoding request, so that nobody has to be preempted.  A request
         that turns out to have ended on its token (eos, a stop sequence) has then run once too often, and that
         result is dropped.  In every other case this returns None and changes nothing: the caller waits for
-        the running batch and schedules as usual."""
+        the running batch and schedules as usual.
+
+        One more way to None: all the checks pass, the running batch's effects are applied (cached lengths,
+        placeholders) and the ordinary ``schedule`` then finds nothing to run, because every request that is left
+        reaches its token count in ``running_batch`` and nobody waits.  The requests then already end in
+        placeholders; ``postprocess(running_batch, tokens)`` overwrites them as it does after a step launched
+        ahead, so the caller still only has to wait for the running batch and go on."""
         items = running_batch.items
         if self._rejected or not items:
             return None

@@ -18,7 +18,7 @@ import json
 import os
 import sys
 
-PAGE_SIZE = 16
+DEFAULT_PAGE_SIZE = 16    # the reference's --block-size default (atom/model_engine/arg_utils.py)
 
 
 def main(argv=None) -> int:
@@ -29,9 +29,14 @@ def main(argv=None) -> int:
     parser.add_argument("--out", required=True, help="folder for the <step>.f32 files")
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="the most tokens live requests hold at any time (each rounded up to 64)")
+    parser.add_argument("--block-size", type=int, default=DEFAULT_PAGE_SIZE,
+                        help="tokens a cache page holds")
     parser.add_argument("--max-requests", type=int, default=8, help="state slots (live requests at a time)")
     parser.add_argument("--enforce-eager", action="store_true", help="never replay captured HIP graphs")
     args = parser.parse_args(argv)
+    page_size = args.block_size
+    if page_size <= 0:
+        parser.error("--block-size must be positive")
 
     def say(msg):
         print(f"[trace_run] {msg}", file=sys.stderr, flush=True)
@@ -48,12 +53,12 @@ def main(argv=None) -> int:
     ops = HipKernels(device)   # builds the kernel library on first use
     say(f"kernel library {ops.path}")
     model, _ = load_model(args.model, dtype=dtype, device=device, progress=say)
-    num_pages = max(1, -(-args.max_tokens // PAGE_SIZE))
-    core = build_core(model, ops, dtype=dtype, device=device, page_size=PAGE_SIZE, num_pages=num_pages,
+    num_pages = max(1, -(-args.max_tokens // page_size))
+    core = build_core(model, ops, dtype=dtype, device=device, page_size=page_size, num_pages=num_pages,
                       max_num_seqs=args.max_requests,
                       graph_sizes=None if args.enforce_eager else [1, 2, 4, 8])
     os.makedirs(args.out, exist_ok=True)
-    say(f"ready: {num_pages} pages of {PAGE_SIZE} tokens per group, {args.dtype}")
+    say(f"ready: {num_pages} pages of {page_size} tokens per group, {args.dtype}")
 
     for line in sys.stdin:
         line = line.strip()

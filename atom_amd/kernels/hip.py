@@ -713,10 +713,14 @@ class HipKernels:
             # histograms of the threshold search: zero when made, and left zero by every call
             need = rows * (4096 * 12 + 32)
             ws_filter = self._zeroed.get("sample_filter")
-            if ws_filter is None or ws_filter.numel() < need or torch.cuda.is_current_stream_capturing():
+            if ws_filter is None or ws_filter.numel() < need:
+                if torch.cuda.is_current_stream_capturing():
+                    # making it would record a fill node into the graph; the caller samples these rows once
+                    # outside a capture first, which leaves the workspace in place
+                    raise KernelError("sample: the top-k / top-p workspace has to exist before a graph is captured "
+                                      f"({rows} rows need {need} bytes)")
                 ws_filter = torch.zeros(need, dtype=torch.uint8, device=self.device)
-                if not torch.cuda.is_current_stream_capturing():
-                    self._zeroed["sample_filter"] = ws_filter
+                self._zeroed["sample_filter"] = ws_filter
         self._done("sample", self.lib.atom_sample(
             _ptr(logits), _ptr(temperatures), _ptr(top_ks), _ptr(top_ps), _ptr(noise), ctypes.c_long(stride),
             _ptr(seeds), _ptr(counters), _ptr(out), rows, vocab, ctypes.c_float(eps), _ptr(ws_vals), _ptr(ws_idx),

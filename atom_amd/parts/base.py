@@ -153,6 +153,11 @@ class Mixer(Part):
         registered cache kind (``cache.kinds.register_cache_kind``), or None."""
         return None
 
+    def page_size_problem(self, page_size: int) -> str | None:
+        """Why this mixer's kernels cannot work with cache pages of ``page_size`` tokens, or None if they can.
+        Asked when the cache is planned, so that a page size is refused before anything is allocated."""
+        return None
+
     def step_key(self):
         """Mixers that return equal keys (hashable, not None) share one ``prepare_step`` a step; None:
         this mixer prepares nothing."""

@@ -10,6 +10,10 @@ engine's own step loop (scheduler, step function, sampler).  ``value`` is decode
 a second.  It also times one 2,048-token prefill and decoding at batch 1 and 64, and
 prints one JSON line.  More than one GPU is not built: ``--gpus N>1`` says so and exits 2.
 
+With no ``--shape`` the same run goes on to the other shapes' workloads (below), the reference's two
+single-stream pairs, and the 8B shape at 16,384 and 32,768 tokens of context, and adds their records
+under ``shapes`` (their headline numbers also under ``points``).
+
 ``--shape 4b`` runs the Qwen3-4B shape (hidden 2560 under 32 heads of 128, tied head) on its
 workload: 32 requests with prompts of 64 to 3,072 tokens through the scheduler, prompt portions
 of 512 tokens beside the running requests' decode tokens, 128 output tokens each.
@@ -242,14 +246,137 @@ def run_long(llm, args, name, raw, layers, gen, batch: int = 16, prompt_len: int
     }
 
 
+def make_engine(args, shape_key: str, *, max_seqs: int, max_model_len: int, pages: int, budget: int, layers=None):
+    """The engine on a shape's sizes with seeded random weights; returns (engine, name, raw config, layers, generator)."""
+    import torch
+
+    from atom_amd import LLMEngine
+    from atom_amd.config import model_config_from_dict
+
+    name, shape, seed = SHAPES[shape_key]
+    raw = dict(shape)
+    layers = layers or raw["num_hidden_layers"]
+    raw["num_hidden_layers"] = layers
+    t0 = time.time()
+    llm = LLMEngine(f"{name.lower()}-random", model_config=model_config_from_dict(raw), load_dummy="random", seed=seed,
+                    dtype="bf16", max_model_len=max_model_len, kv_cache_block_size=16, num_kvcache_blocks=pages,
+                    max_num_seqs=max_seqs, max_num_batched_tokens=budget, enforce_eager=args.enforce_eager,
+                    deferred_output=not args.no_deferred_output,
+                    cudagraph_capture_sizes=[s for s in (1, 2, 4, 8, 16, 32, 48, 64, 128, 256) if s <= max_seqs])
+    torch.cuda.synchronize()
+    print(f"[bench] {name} shape ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    raw["num_hidden_layers"] = SHAPES[shape_key][1]["num_hidden_layers"]
+    return llm, name, raw, layers, torch.Generator().manual_seed(seed)
+
+
+def release(llm) -> None:
+    """Gives an engine's device memory (weights, cache, graphs) back before the next one is built."""
+    import gc
+
+    import torch
+
+    if llm.core.graphs is not None:
+        llm.core.graphs.captured.clear()
+    llm.core = llm.model = llm.scheduler = llm.sampler = None
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def time_prefill(llm, raw, layers, gen, tokens: int, repeats: int = 3) -> dict:
+    """One prompt of ``tokens`` tokens through ``generate`` with one output token: the best of ``repeats``."""
+    import torch
+    from atom_amd import SamplingParams
+
+    sp = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
+    vocab = raw["vocab_size"]
+    llm.generate([torch.randint(0, vocab, (tokens,), generator=gen).tolist()], sp)   # warm-up: library autotuning
+    times = []
+    for _ in range(repeats):
+        p = torch.randint(0, vocab, (tokens,), generator=gen).tolist()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        llm.generate([p], sp)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t)
+    best = min(times)
+    flops = prefill_flops(raw, layers, tokens)
+    return {"value": round(tokens / best, 1), "tokens": tokens, "ms": round(best * 1e3, 3),
+            "frac": round(flops / best / MFMA_PEAK["bf16"], 4)}
+
+
+def time_decode(llm, args, raw, gen, batch: int, context: int, steps: int, warmup: int):
+    """``batch`` requests of ``context`` random prompt tokens, prefilled untimed, then ``steps`` timed decode steps
+    through the engine's own loop.  Returns (seconds, context length at the first timed step)."""
+    import torch
+    from atom_amd import SamplingParams
+
+    # prompts are admitted over several steps, so the first requests are some tokens ahead of the last
+    # when all decode: leave room, so that none finishes (and the batch does not shrink) while timed
+    admission_steps = -(-batch * context // llm.config.max_num_batched_tokens) + batch
+    sp = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, seed=1,
+                        max_tokens=steps + warmup + admission_steps + 2, ignore_eos=True)
+    for _ in range(batch):
+        llm.add_request(torch.randint(0, raw["vocab_size"], (context,), generator=gen).tolist(), sp)
+    while any(s.num_completion_tokens == 0 for s in llm.seqs.values()):   # prompts, untimed
+        llm.step()
+    for _ in range(warmup):
+        llm.step()
+    torch.cuda.synchronize()
+    assert len(llm.scheduler.running) == batch and not llm.scheduler.waiting
+    start_ctx = next(iter(llm.seqs.values())).num_tokens
+    t = time.perf_counter()
+    for _ in range(steps):
+        llm.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t
+    assert len(llm.scheduler.running) == batch, "a request finished inside the timed steps"
+    while not llm.is_finished():
+        llm.step()
+    llm.seqs.clear()
+    return elapsed, start_ctx
+
+
+def decode_roofline(raw, layers, batch, ctx0, steps, elapsed) -> dict:
+    step_bytes = weight_bytes(raw, layers) + batch * (ctx0 + steps / 2) * kv_bytes_per_token(raw, layers)
+    achieved = step_bytes * steps / elapsed
+    return {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK, 4)}
+
+
+def run_long_context(args, contexts=(16384, 32768), batch: int = 8, prefill_tokens: int = 16384) -> dict:
+    """The 8B shape far from the headline's context: decode at ``batch`` requests of 16,384 and 32,768 tokens each,
+    and one prompt of 16,384 tokens prefilled in one step."""
+    longest = max(contexts)
+    max_model_len = longest + 1024
+    llm, name, raw, layers, gen = make_engine(args, "8b", max_seqs=batch, max_model_len=max_model_len,
+                                              pages=batch * max_model_len // 16, budget=16384)
+    out = {"config": flat_config(name, raw, layers, global_batch=batch, seq_len=longest, max_model_len=max_model_len,
+                                 hip_graphs=not args.enforce_eager), "decode": {}}
+    steps = min(args.steps, 32)
+    for context in contexts:
+        elapsed, ctx0 = time_decode(llm, args, raw, gen, batch, context, steps, args.warmup)
+        roof = decode_roofline(raw, layers, batch, ctx0, steps, elapsed)
+        out["decode"][f"ctx{context}"] = {"value": round(batch * steps / elapsed, 1), "ms_per_step": round(elapsed / steps * 1e3, 4),
+                                          "roofline": roof}
+        print(f"[bench] decode batch {batch} at context {context}: {elapsed / steps * 1e3:.3f} ms/step, "
+              f"{roof['frac']} of the HBM peak", file=sys.stderr, flush=True)
+    last = out["decode"][f"ctx{longest}"]
+    out["ms_per_step"], out["roofline"] = last["ms_per_step"], last["roofline"]
+    out["prefill"] = time_prefill(llm, raw, layers, gen, prefill_tokens, repeats=2)
+    print(f"[bench] prefill {out['prefill']}", file=sys.stderr, flush=True)
+    release(llm)
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
+    ap.add_argument("--shape", choices=sorted(SHAPES), default=None,
                     help="8b: decode at batch 8 (and 1, 64) and a 2,048-token prefill; 4b: 32 mixed requests; "
-                         "32b: 8,192-token prompts in portions, then decode at batch 16 with the cache sized from memory")
+                         "32b: 8,192-token prompts in portions, then decode at batch 16 with the cache sized from memory; "
+                         "not given: the 8b run, and the other shapes' workloads beside it under 'shapes'")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
     ap.add_argument("--max-model-len", type=int, default=None,
@@ -278,141 +405,99 @@ def main() -> int:
 
     import logging
 
-    import torch
-
-    from atom_amd import LLMEngine, SamplingParams
-    from atom_amd.config import model_config_from_dict
-
     logging.basicConfig(level=logging.INFO, stream=sys.stderr, format="[bench] %(name)s: %(message)s")
     logging.getLogger("atom_amd").setLevel(logging.INFO if args.shape == "32b" else logging.WARNING)
-    name, shape, seed = SHAPES[args.shape]
-    raw = dict(shape)
-    full_layers = raw["num_hidden_layers"]
-    layers = args.layers or full_layers
-    raw["num_hidden_layers"] = layers
-    cfg = model_config_from_dict(raw)
+    # no shape named, nothing else asked for: the headline run and every other shape's workload beside it
+    everything = args.shape is None and not (args.single or args.mixed or args.decode or args.layers)
+    args.shape = args.shape or "8b"
+    line = run_shape(args)
+    if everything:
+        line["shapes"] = shapes = {}
+        for key, sub in (("qwen3_4b_mixed", dict(shape="4b")), ("qwen3_32b_long", dict(shape="32b")),
+                         ("qwen3_8b_single", dict(shape="8b", single="18,80;549,256"))):
+            sub_args = argparse.Namespace(**{**vars(args), **sub, "steps": min(args.steps, 32) if key == "qwen3_32b_long" else args.steps})
+            shapes[key] = run_shape(sub_args)
+        shapes["qwen3_8b_long_context"] = run_long_context(args)
+        # the same numbers flat, beside the headline's other points
+        pts = line["points"]
+        pts["mixed_4b_output_tok_s"] = shapes["qwen3_4b_mixed"]["value"]
+        pts["decode_32b_b16_ctx8192"] = shapes["qwen3_32b_long"]["value"]
+        pts["prefill_32b_tok_s"] = shapes["qwen3_32b_long"]["prefill"]["value"]
+        for pair, row in shapes["qwen3_8b_single"]["single_stream"].items():
+            pts[f"single_{pair}_ttft_ms"], pts[f"single_{pair}_tpot_ms"] = row["ttft_ms"], row["tpot_ms"]
+        for ctx, row in shapes["qwen3_8b_long_context"]["decode"].items():
+            pts[f"decode_b8_{ctx}"] = row["value"]
+            line["points_roofline"][f"decode_b8_{ctx}"] = row["roofline"]["frac"]
+        pts["prefill_16384_tok_s"] = shapes["qwen3_8b_long_context"]["prefill"]["value"]
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+def run_shape(args) -> dict:
+    """One shape's workload on an engine of its own; returns the record of that run."""
+    mixed_requests = 0 if (args.single or args.decode) else (args.mixed or (32 if args.shape == "4b" else 0))
     plain = bool(args.single) or args.decode
-    mixed = 0 if plain else (args.mixed or (32 if args.shape == "4b" else 0))
-    long_run = args.shape == "32b" and not mixed and not plain
+    long_run = args.shape == "32b" and not mixed_requests and not plain
     points = sorted({int(x) for x in args.points.split(",") if x} | {args.batch})
-    block = 16
     if long_run:
         max_seqs, max_model_len, pages, budget = 16, args.max_model_len or 8192 + 512, -1, 4096
     else:
-        max_seqs = max(points + [mixed])
+        max_seqs = max(points + [mixed_requests])
         max_model_len = args.max_model_len or max(4096, 2 * args.context)
-        pages, budget = max_seqs * max_model_len // block, (512 + mixed if mixed else 16384)
+        pages, budget = max_seqs * max_model_len // 16, (512 + mixed_requests if mixed_requests else 16384)
     budget = args.budget or budget
-    t0 = time.time()
-    llm = LLMEngine(f"{name.lower()}-random", model_config=cfg, load_dummy="random", seed=seed, dtype="bf16",
-                    max_model_len=max_model_len, kv_cache_block_size=block, num_kvcache_blocks=pages,
-                    max_num_seqs=max_seqs, max_num_batched_tokens=budget, enforce_eager=args.enforce_eager,
-                    deferred_output=not args.no_deferred_output,
-                    cudagraph_capture_sizes=[s for s in (1, 2, 4, 8, 16, 32, 48, 64, 128, 256) if s <= max_seqs])
-    torch.cuda.synchronize()
-    print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
-    gen = torch.Generator().manual_seed(seed)
-    vocab = raw["vocab_size"]
+    llm, name, raw, layers, gen = make_engine(args, args.shape, max_seqs=max_seqs, max_model_len=max_model_len,
+                                              pages=pages, budget=budget, layers=args.layers)
+    try:
+        if args.single:
+            pairs = [tuple(int(v) for v in pair.split(",")) for pair in args.single.split(";")]
+            return run_single(llm, args, name, raw, layers, gen, pairs)
+        if mixed_requests:
+            return run_mixed(llm, args, name, raw, layers, gen, mixed_requests)
+        if long_run:
+            return run_long(llm, args, name, raw, layers, gen)
+        return run_points(llm, args, name, raw, layers, gen, points, max_model_len)
+    finally:
+        release(llm)
 
-    def prompt():
-        return torch.randint(0, vocab, (args.context,), generator=gen).tolist()
 
-    def sync():
-        torch.cuda.synchronize()
-
-    if args.single:
-        pairs = [tuple(int(v) for v in pair.split(",")) for pair in args.single.split(";")]
-        print(json.dumps(run_single(llm, args, name, raw, layers, gen, pairs)), flush=True)
-        return 0
-    if mixed:
-        print(json.dumps(run_mixed(llm, args, name, raw, layers, gen, mixed)), flush=True)
-        return 0
-    if long_run:
-        print(json.dumps(run_long(llm, args, name, raw, layers, gen)), flush=True)
-        return 0
-
-    # ---- prefill of one 2,048-token prompt
+def run_points(llm, args, name, raw, layers, gen, points, max_model_len) -> dict:
+    """A prefill of ``--context`` tokens and decode at every batch size of ``points``."""
     prefill = None
     if not args.no_prefill:
-        sp = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
-        llm.generate([prompt()], sp)            # warm-up: library autotuning, first-use allocations
-        times = []
-        for _ in range(3):
-            p = prompt()
-            sync()
-            t = time.perf_counter()
-            llm.generate([p], sp)
-            sync()
-            times.append(time.perf_counter() - t)
-        best = min(times)
-        flops = prefill_flops(raw, layers, args.context)
-        prefill = {"value": round(args.context / best, 1), "tokens": args.context, "ms": round(best * 1e3, 3),
-                   "frac": round(flops / best / MFMA_PEAK["bf16"], 4)}
+        prefill = time_prefill(llm, raw, layers, gen, args.context)
         print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
-
-    # ---- decode at each batch size
-    def decode(batch: int, steps: int, warmup: int):
-        # prompts are admitted over several steps, so the first requests are some tokens ahead of the last
-        # when all decode: leave room, so that none finishes (and the batch does not shrink) while timed
-        admission_steps = -(-batch * args.context // 16384) + 1
-        sp = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, seed=1,
-                            max_tokens=steps + warmup + admission_steps + 2, ignore_eos=True)
-        for _ in range(batch):
-            llm.add_request(prompt(), sp)
-        while any(s.num_completion_tokens == 0 for s in llm.seqs.values()):   # prompts, untimed
-            llm.step()
-        for _ in range(warmup):
-            llm.step()
-        sync()
-        assert len(llm.scheduler.running) == batch and not llm.scheduler.waiting
-        start_ctx = next(iter(llm.seqs.values())).num_tokens
-        t = time.perf_counter()
-        for _ in range(steps):
-            llm.step()
-        sync()
-        elapsed = time.perf_counter() - t
-        assert len(llm.scheduler.running) == batch, "a request finished inside the timed steps"
-        while not llm.is_finished():
-            llm.step()
-        llm.seqs.clear()
-        return elapsed, start_ctx
-
     results = {}
     for b in points:
         steps = args.steps
-        elapsed, ctx0 = decode(b, steps, args.warmup)
+        elapsed, ctx0 = time_decode(llm, args, raw, gen, b, args.context, steps, args.warmup)
         results[b] = (elapsed, ctx0, steps)
         print(f"[bench] decode batch {b}: {b * steps / elapsed:.1f} tok/s, {elapsed / steps * 1e3:.3f} ms/step",
               file=sys.stderr, flush=True)
 
     def roofline(b):
         elapsed, ctx0, steps = results[b]
-        step_bytes = weight_bytes(raw, layers) + b * (ctx0 + steps / 2) * kv_bytes_per_token(raw, layers)
-        return step_bytes * steps / elapsed
+        return decode_roofline(raw, layers, b, ctx0, steps, elapsed)
 
     elapsed, ctx0, steps = results[args.batch]
-    per_step = elapsed / steps
-    achieved = roofline(args.batch)
     line = {
         "metric": f"decode tok/s at batch {args.batch} ({name}, bf16); prefill tok/s at {args.context} tokens and "
                   f"batch {'/'.join(str(b) for b in points if b != args.batch)} alongside",
         "value": round(args.batch * steps / elapsed, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
-        "warmup": args.warmup, "ms_per_step": round(per_step * 1e3, 4), "higher_is_better": True,
+        "warmup": args.warmup, "ms_per_step": round(elapsed / steps * 1e3, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic: seeded uniform random token ids, seeded random N(0, 0.02) weights",
         "config": flat_config(name, raw, layers, global_batch=args.batch, seq_len=args.context,
                               max_model_len=max_model_len, decode_steps=steps, hip_graphs=not args.enforce_eager,
                               deferred_output=not args.no_deferred_output),
-        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK, 4)},
+        "roofline": roofline(args.batch),
         "points": {f"decode_b{b}": round(b * results[b][2] / results[b][0], 2) for b in points if b != args.batch},
         # the same fraction of the HBM peak for the other batch sizes
-        "points_roofline": {f"decode_b{b}": round(roofline(b) / HBM_PEAK, 4) for b in points if b != args.batch},
+        "points_roofline": {f"decode_b{b}": roofline(b)["frac"] for b in points if b != args.batch},
     }
     if prefill:
         line["prefill"] = prefill
-    print(json.dumps(line), flush=True)
-    return 0
+    return line
 
 
 if __name__ == "__main__":

@@ -178,10 +178,10 @@ def run_in_process(core, steps: list[dict]) -> dict[int, torch.Tensor]:
 
 
 def run_program(model_dir: str, dtype: str, steps: list[dict], out_dir: str, max_tokens: int, vocab: int,
-                env: dict | None = None, timeout: int = 600) -> dict[int, torch.Tensor]:
+                env: dict | None = None, timeout: int = 600, extra: list[str] | None = None) -> dict[int, torch.Tensor]:
     """Drives ``bin/trace_run``: one step a line, waiting for its ``done`` before the next."""
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
-           "--out", out_dir, "--max-tokens", str(max_tokens)]
+           "--out", out_dir, "--max-tokens", str(max_tokens), *(extra or [])]
     proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, env=env)
     try:
         for s in steps:

@@ -90,7 +90,7 @@ def test_engine_config(tmp_path):
     with pytest.raises(ConfigError):
         Config("x", model_config=mc, dtype="fp8")
     with pytest.raises(ConfigError):
-        Config("x", model_config=mc, kv_cache_block_size=10)
+        Config("x", model_config=mc, kv_cache_block_size=0)
     with pytest.raises(ConfigError):
         Config("x", model_config=mc, long_prefill_token_threshold=4)
     with pytest.raises(ConfigError):
@@ -129,3 +129,23 @@ def test_cli_graph_sizes_for_steps_with_prompt_portions():
     off = EngineArgs.from_cli_args(parser.parse_args(["--model", "m"]))._get_engine_kwargs()
     on = EngineArgs.from_cli_args(parser.parse_args(["--model", "m", "--cudagraph-prefill-sizes", "[256, 512]"]))
     assert off["cudagraph_prefill_sizes"] == [] and on._get_engine_kwargs()["cudagraph_prefill_sizes"] == [256, 512]
+
+
+def test_cli_renders_prompts_through_the_chat_template(tmp_path):
+    """With a tokenizer that has a chat template the command line sends one user message with the generation
+    prompt appended (atom/examples/simple_inference.py:66-70); without a template, the text itself."""
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    from transformers import PreTrainedTokenizerFast
+
+    from atom_amd.examples.simple_inference import render_chat
+
+    words = ["<|im_start|>", "<|im_end|>", "user", "assistant", "1+2+3=?", "[UNK]"]
+    raw = Tokenizer(models.WordLevel({w: i for i, w in enumerate(words)}, unk_token="[UNK]"))
+    raw.pre_tokenizer = pre_tokenizers.WhitespaceSplit()
+    tok = PreTrainedTokenizerFast(tokenizer_object=raw, unk_token="[UNK]")
+    assert render_chat(tok, "1+2+3=?") == "1+2+3=?"
+    tok.chat_template = ("{% for m in messages %}<|im_start|> {{ m['role'] }} {{ m['content'] }} <|im_end|> {% endfor %}"
+                         "{% if add_generation_prompt %}<|im_start|> assistant{% endif %}")
+    text = render_chat(tok, "1+2+3=?")
+    assert text == "<|im_start|> user 1+2+3=? <|im_end|> <|im_start|> assistant"
+    assert tok.encode(text) == [0, 2, 4, 1, 0, 3]

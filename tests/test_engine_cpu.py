@@ -4,6 +4,7 @@ must reproduce the plain implementation under every way of cutting the work.  Wh
 tested here is paging, batching and metadata; the kernels themselves are tested on the GPU."""
 
 import pytest
+import torch
 
 import replay
 from helpers import make_core, oracle_logits, random_ids
@@ -64,6 +65,30 @@ def test_layer_order_is_data():
     replay.check(steps, results, requests, {"x": want}, "float32", "order")
     plain = oracle_logits("B", ids)
     assert (plain - want).abs().max() > 1e-3, "the changed order must change the result"
+
+
+def test_a_mixer_may_refuse_a_page_size():
+    """What a page size must be is the mixers' to say: the cache plan asks each of them."""
+    from atom_amd.parts.attention import GroupedQueryAttention
+
+    core = make_core("A", "float32", PlainKernels(), "cpu", page_size=6)     # attention takes any positive size
+    ids = random_ids("A", 20, 1)
+    from atom_amd.engine.core import StepEntry
+    logits = core.step([StepEntry("a", ids, [19])])
+    assert replay.first_bad({19: logits[0]}, oracle_logits("A", ids), "float32") is None
+
+    class Picky(GroupedQueryAttention):
+        def page_size_problem(self, page_size):
+            return None if page_size % 32 == 0 else "this mixer's kernels read 32 keys at a time"
+
+    core.model.blocks[1].mixer.__class__ = Picky
+    try:
+        with pytest.raises(ValueError, match="pages of 16 tokens do not suit layer 1 .Picky.: this mixer's kernels"):
+            from atom_amd.cache.storage import plan_cache
+            plan_cache(core.model, 16, torch.float32, num_pages=4)
+        plan_cache(core.model, 64, torch.float32, num_pages=4)
+    finally:
+        core.model.blocks[1].mixer.__class__ = GroupedQueryAttention
 
 
 def test_step_rejects_bad_input():

@@ -33,6 +33,48 @@ def test_graph_cuts_match_plain(which, cut, dtype):
     replay.check(steps, results, requests, oracle, dtype, f"graph/{which}/{cut}/{dtype}")
 
 
+ORDERS = {"C": [(0, None), (1, None), (1, None), (2, 1), (3, 0)],   # a windowed and a full run that read
+          "D": [(0, None), (1, None), (1, None), (0, 0)]}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["C", "D"])
+@pytest.mark.parametrize("cut", ["tail", "mixed"])
+def test_an_order_whose_runs_share_and_read_caches(which, cut, dtype):
+    """The running order as data, on the GPU kernels and through replayed graphs: a layer run twice, each run
+    with a cache of its own, and runs that read an earlier run's cache and write none (in the decode steps of
+    few rows that is the kernel that norms, rotates, writes and attends in one, with its write switched off)."""
+    order = ORDERS[which]
+    requests = _requests(which)
+    oracle = {rid: oracle_logits(which, ids, order=order) for rid, ids in requests.items()}
+    first = next(iter(requests))
+    assert (oracle_logits(which, requests[first]) - oracle[first]).abs().max() > 1e-3, "the order must matter"
+    steps = replay.tail(requests) if cut == "tail" else replay.mixed(requests, seed=11, decode_tail=20)
+    pages = -(-replay.peak_tokens(steps, 64) // 16)
+    core = make_core(which, dtype, gpu_ops(), "cuda:0", num_pages=pages, page_size=16, graph_sizes=[1, 2, 4],
+                     order=order)
+    assert core.graphs is not None
+    results = replay.run_in_process(core, steps)
+    assert core.graphs.replays >= 20
+    replay.check(steps, results, requests, oracle, dtype, f"order/{which}/{cut}/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_that_do_not_divide_the_longest_context(dtype):
+    """Pages of 24 tokens and 2,048 positions: the graphs' block tables name more positions than the rotation
+    tables hold, which must refuse no capture and change no logit."""
+    which = "D"
+    requests = {f"q{k}": random_ids(which, n, 300 + k) for k, n in enumerate([50, 131, 75])}
+    oracle = {rid: oracle_logits(which, ids) for rid, ids in requests.items()}
+    steps = replay.tail(requests)
+    pages = -(-replay.peak_tokens(steps, 72) // 24)
+    core = make_core(which, dtype, gpu_ops(), "cuda:0", num_pages=pages, page_size=24, graph_sizes=[1, 2])
+    assert core.graphs is not None and core.graphs.widths[0] * 24 > 2048
+    results = replay.run_in_process(core, steps)
+    assert core.graphs.replays >= 90
+    replay.check(steps, results, requests, oracle, dtype, f"page24/{dtype}")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("which", ["B", "C", "D"])
 def test_steps_with_prompt_portions_replayed_as_graphs(which, dtype):

@@ -148,7 +148,7 @@ def test_float32_logits_keep_their_precision_with_many_rows():
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hq,hkv,d,rot,page", [(4, 2, 16, 16, 16), (6, 3, 32, 32, 8), (5, 5, 48, 24, 4),
                                               (8, 1, 128, 128, 32), (3, 1, 80, 0, 16), (5, 2, 64, 64, 16),
-                                              (2, 1, 256, 256, 8), (3, 3, 96, 96, 16)])
+                                              (2, 1, 256, 256, 8), (3, 3, 96, 96, 16), (4, 2, 64, 64, 6)])
 @pytest.mark.parametrize("norm", [True, False])
 @pytest.mark.parametrize("tokens", [11, 45])   # 32 tokens and more take the vector kernel where it applies
 def test_qk_norm_rope_kv_write(dtype, hq, hkv, d, rot, page, norm, tokens):
@@ -263,7 +263,7 @@ def _attention_case(dtype, hq, hkv, d, page, window, q_lens, ctx_lens, seed, sca
 
 ATTN_SHAPES = [  # hq, hkv, d, page
     (4, 2, 16, 16), (6, 3, 32, 8), (8, 2, 64, 16), (5, 5, 96, 4), (32, 8, 128, 16), (3, 1, 256, 32), (40, 2, 64, 16),
-    (2, 1, 48, 16), (7, 7, 80, 8),
+    (2, 1, 48, 16), (7, 7, 80, 8), (4, 2, 64, 6), (8, 2, 128, 10),   # the last two: pages no matrix-core kernel takes
 ]
 
 

@@ -88,6 +88,20 @@ def test_trace_run_program(which, dtype, tmp_path):
     replay.check(steps, out, requests, oracle, dtype, f"trace_run/{which}/{dtype}")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program_with_its_own_page_size(dtype, tmp_path):
+    """``bin/trace_run --block-size 8``: config B's own pages through the program, two live requests at a
+    time in a pool that holds far less than what runs through it."""
+    requests = _requests("B", seed=5)
+    oracle = _oracle("B", requests)
+    steps = replay.mixed(requests, seed=6, max_live=2)
+    peak = replay.peak_tokens(steps, 64)
+    assert sum(len(v) for v in requests.values()) > 1.3 * peak      # pages are used again
+    out = replay.run_program(tiny_folder("B"), dtype, steps, str(tmp_path / "out"), peak, CONFIGS["B"]["vocab_size"],
+                             extra=["--block-size", "8"])
+    replay.check(steps, out, requests, oracle, dtype, f"trace_run/B/page8/{dtype}")
+
+
 def test_trace_run_wants_nothing(tmp_path):
     """Steps that want nothing write no file; a request may sit out steps and go on later."""
     ids = random_ids("A", 40, 5)

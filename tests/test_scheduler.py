@@ -394,6 +394,22 @@ def test_schedule_ahead_skips_a_request_at_its_last_token():
     core.manager.check()
 
 
+def test_schedule_ahead_with_nothing_left_to_run_leaves_placeholders_that_postprocess_fills():
+    """Every request of the running batch reaches its token count in it and nobody waits: the effects of the
+    running batch are applied, nothing is scheduled, and the tokens still land where they belong."""
+    sched, core = make(blocks=40, block=4)
+    (a,) = _decoding(sched, [6], max_tokens=2, ignore_eos=True)
+    running = sched.schedule()
+    assert [it.seq.id for it in running.items] == [a.id]
+    assert sched.schedule_ahead(running) is None
+    assert a.awaits_token and a.num_cached_tokens == 7      # not "nothing changed": the request ends in a placeholder
+    done = sched.postprocess(running, {a.id: 55})
+    assert [s.id for s in done] == [a.id] and a.leave_reason == "max_tokens"
+    assert a.token_ids[-1] == 55 and not a.awaits_token and a.num_completion_tokens == 2
+    assert a.id not in core.manager and sched.schedule() is None
+    core.manager.check()
+
+
 def test_schedule_ahead_admits_and_continues_prompts():
     """What a step scheduled ahead may hold besides decode tokens: a request admitted meanwhile, the next
     portion of an unfinished prompt; a prompt that ends in the running batch decodes in the next."""
