@@ -799,11 +799,18 @@ static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
 // dimension of one step of the second product, in the order (4 g + i, 16 + 4 g + i) that the first product
 // leaves them in a lane.
 //
+// With KS = 2 the block has eight waves: the second four are the same heads and tokens again, and the two
+// halves take the key tiles in turn (tile 0, 2, 4 .. and 1, 3, 5 ..), each with LDS tiles of its own, and add
+// their results at the end through LDS.  A block then keeps two waves on every SIMD for as long as it runs, one
+// in its products while the other is in its softmax; a block of four waves only has that while another block
+// shares its CU, and the longest blocks of a causal prompt, which decide how long the launch takes, run mostly
+// after their shorter neighbours have left.
+//
 // Needs D % 64 == 0 and page_size % 8 == 0.
 constexpr float kLazyMax = 8.f;
 
-template <int D, int GH, int TK>
-__global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_tiled_kernel(AttnParams p) {
+template <int D, int GH, int TK, int KS>
+__global__ void __launch_bounds__(256 * KS, (D <= 128 && KS == 1 ? 2 : 1)) attention_prefill_tiled_kernel(AttnParams p) {
   constexpr int KCH = D / 32;
   constexpr int DT = D / 16;
   constexpr int RT = 2;
@@ -811,9 +818,19 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
   constexpr int KSTR = D + 8;            // LDS row of a key, in elements: rows start 4 banks apart
   constexpr int VSTR = TK + 8;           // LDS row of V^T (one d), in elements: 16-byte aligned, rows 4 banks apart
   constexpr int PT = D * TK / 8 / 256;   // 16-byte pieces of each tile that a thread moves
-  __shared__ __attribute__((aligned(16))) bf16_t ks[TK * KSTR];
-  __shared__ __attribute__((aligned(16))) bf16_t vs[D * VSTR];
-  const int tid = threadIdx.x;
+#ifndef ATOM_PF_AHEAD
+#define ATOM_PF_AHEAD 4
+#endif
+
+  constexpr int AHEAD = ATOM_PF_AHEAD;   // operands read from LDS ahead of the product that takes them
+  constexpr int TILE_ELEMS = TK * KSTR + D * VSTR;   // a K tile and a V^T tile
+  constexpr int NS = RT * DT * 4 + 2 * RT;           // floats a lane hands over when the halves are added
+  constexpr int SMEM_TILES = KS * TILE_ELEMS * 2, SMEM_SUMS = KS > 1 ? 4 * NS * kWave * 4 : 0;
+  __shared__ __attribute__((aligned(16))) char smem[SMEM_TILES > SMEM_SUMS ? SMEM_TILES : SMEM_SUMS];
+  const int part = threadIdx.x / 256;    // which half of the key tiles (always 0 with KS = 1)
+  const int tid = threadIdx.x % 256;
+  bf16_t* const ks = reinterpret_cast<bf16_t*>(smem) + part * TILE_ELEMS;
+  bf16_t* const vs = ks + TK * KSTR;
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
   const int r16 = lane & 15;
@@ -827,10 +844,16 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
   // item down while its second half walks it from the shortest up, so that the two blocks that meet on a
   // CU (block b and block b + n / 2, as blocks are handed out in order) are a long and a short one.
   // Larger heads run one block a CU, which takes tile b and then tile n - 1 - b.
+  // Blocks of eight waves run one a CU and take the items in the order of the list, longest first.
   constexpr bool TWO = D <= 128;
   for (int pass = 0; pass < 2; ++pass) {
   int tile, ygroup;
-  if (TWO) {
+  if (KS > 1) {
+    if (pass == 1) break;
+    const int groups = p.hq / GH;
+    tile = (int)blockIdx.x / groups;
+    ygroup = (int)blockIdx.x - tile * groups;
+  } else if (TWO) {
     if (pass == 1) break;
     const int total = gridDim.x, half = (total + 1) / 2, groups = p.hq / GH;
     const int item = (int)blockIdx.x < half ? (int)blockIdx.x : total - 1 - ((int)blockIdx.x - half);
@@ -948,18 +971,20 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
     }
   };
 
-  if (kb < ke) {
-    pages_of(kb);
-    load_tile(kb);
-    if (kb + TK < ke) pages_of(kb + TK);
+  constexpr int STEP = KS * TK;          // keys the block walks at a time
+  if (kb + part * TK < ke) {
+    pages_of(kb + part * TK);
+    load_tile(kb + part * TK);
+    if (kb + part * TK + STEP < ke) pages_of(kb + part * TK + STEP);
   }
-  for (int k0 = kb; k0 < ke; k0 += TK) {
+  for (int kk = kb; kk < ke; kk += STEP) {
+    const int k0 = kk + part * TK;       // this half's tile
     __syncthreads();   // the previous tile has been read by every wave
-    store_tile();
+    if (k0 < ke) store_tile();
     __syncthreads();
-    if (k0 + TK < ke) {
-      load_tile(k0 + TK);
-      if (k0 + 2 * TK < ke) pages_of(k0 + 2 * TK);
+    if (k0 + STEP < ke) {
+      load_tile(k0 + STEP);
+      if (k0 + 2 * STEP < ke) pages_of(k0 + 2 * STEP);
     }
     if (nrows == 0 || k0 >= my_ke) continue;   // the whole wave: nothing of this tile is visible to it
 
@@ -969,16 +994,33 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int b = 0; b < KB; ++b) s[rt][b] = f32x4{0.f, 0.f, 0.f, 0.f};
-    // (the head-size chunks outermost: successive products go to different accumulators)
+    // (the head-size chunks outermost: successive products go to different accumulators).  The operand of
+    // product i + AHEAD is read from LDS while product i runs: the order is pinned, because left to itself the
+    // compiler reads every operand just before its product and waits for it.
+    {
+      constexpr int NQK = KCH * KB;
+      auto k_operand = [&](int i) {
+        return *reinterpret_cast<const bf16x8*>(ks + (16 * (i % KB) + r16) * KSTR + 32 * (i / KB) + 8 * g);
+      };
+      bf16x8 kf[AHEAD];
 #pragma unroll
-    for (int j = 0; j < KCH; ++j)
+      for (int i = 0; i < AHEAD; ++i) kf[i] = k_operand(i);
 #pragma unroll
-      for (int b = 0; b < KB; ++b) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks + (16 * b + r16) * KSTR + 32 * j + 8 * g);
+      for (int i = 0; i < NQK; ++i) {
+        __builtin_amdgcn_sched_barrier(0);
+        const bf16x8 a = kf[i % AHEAD];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-          s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q32[rt][j], s[rt][b], 0, 0, 0);
+          s[rt][i % KB] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q32[rt][i / KB], s[rt][i % KB], 0, 0, 0);
+        if (i + AHEAD < NQK) kf[i % AHEAD] = k_operand(i + AHEAD);
       }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    constexpr int NPV = (KB / 2) * DT;
+    auto v_operand = [&](int i) {
+      return *reinterpret_cast<const bf16x8*>(vs + (16 * (i % DT) + r16) * VSTR + 32 * (i / DT) + 8 * g);
+    };
+    bf16x8 vf[AHEAD];
 
     // ---- softmax update; lane holds keys k0 + 16 b + 4 g + i of row r16.  The maximum is taken over the
     //      raw scores and the scale goes into the exponent's multiply-add.  A tile that every row of the
@@ -1044,15 +1086,58 @@ __global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1)) attention_prefill_til
     }
 
     // ---- O^T += V^T P^T, 32 keys a step
+    {
 #pragma unroll
-    for (int h = 0; h < KB / 2; ++h)
+      for (int i = 0; i < AHEAD; ++i) vf[i] = v_operand(i);
 #pragma unroll
-      for (int t = 0; t < DT; ++t) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(vs + (16 * t + r16) * VSTR + 32 * h + 8 * g);
+      for (int i = 0; i < NPV; ++i) {
+        __builtin_amdgcn_sched_barrier(0);
+        const bf16x8 a = vf[i % AHEAD];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-          acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[rt][h], acc[rt][t], 0, 0, 0);
+          acc[rt][i % DT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[rt][i / DT], acc[rt][i % DT], 0, 0, 0);
+        if (i + AHEAD < NPV) vf[i % AHEAD] = v_operand(i + AHEAD);
       }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // ---- the two halves of the key tiles are added: the second hands its sums, maxima and accumulators over
+  //      through LDS, lane by lane (both halves hold the same rows and columns in the same lanes)
+  if constexpr (KS > 1) {
+    if (kb + TK < ke) {      // the same for the whole block: the second half had a tile at all
+      __syncthreads();       // every wave has read its last tiles
+      float* area = reinterpret_cast<float*>(smem) + (size_t)wave * NS * kWave + lane;
+      if (part == 1) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+          for (int t = 0; t < DT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) area[((rt * DT + t) * 4 + i) * kWave] = acc[rt][t][i];
+          area[(RT * DT * 4 + rt) * kWave] = run_max[rt];
+          area[(RT * DT * 4 + RT + rt) * kWave] = run_sum[rt];
+        }
+      }
+      __syncthreads();
+      if (part == 0) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          const float other_max = area[(RT * DT * 4 + rt) * kWave];
+          const float other_sum = area[(RT * DT * 4 + RT + rt) * kWave];
+          const float top = fmaxf(run_max[rt], other_max);
+          const float base = top == -INFINITY ? 0.f : top;
+          const float mine = fast_exp2(run_max[rt] - base), theirs = fast_exp2(other_max - base);
+          run_sum[rt] = run_sum[rt] * mine + other_sum * theirs;
+#pragma unroll
+          for (int t = 0; t < DT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              acc[rt][t][i] = acc[rt][t][i] * mine + area[((rt * DT + t) * 4 + i) * kWave] * theirs;
+        }
+      }
+    }
+    if (part != 0) return;   // nothing follows but the first half's writes
   }
 
   // ---- write: lane holds O[row r16][d = 16 t + 4 g + i]
@@ -1084,16 +1169,25 @@ ATOM_EXPORT int atom_attention_prefill_tile_rows(int d, int page_size, int group
 }
 
 template <int D>
-static int launch_prefill_tiled(const AttnParams& p, int num_tiles, int rows_per_tile, hipStream_t stream) {
+static int launch_prefill_tiled(const AttnParams& p, int num_tiles, int rows_per_tile, bool halves, hipStream_t stream) {
   const int group = p.hq / p.hkv;
   const int gh = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
   if (rows_per_tile != 32 * (4 / gh)) return ATOM_BAD_SHAPE;
   dim3 grid((num_tiles + 1) / 2, p.hq / gh), block(256);
   if (D <= 128) grid = dim3(num_tiles * (p.hq / gh), 1);
   constexpr int TK = D <= 128 ? 64 : 32;
-  if (gh == 4) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 4, TK>), grid, block, 0, stream, p);
-  else if (gh == 2) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 2, TK>), grid, block, 0, stream, p);
-  else hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 1, TK>), grid, block, 0, stream, p);
+  if constexpr (D <= 128) {
+    if (halves) {   // eight waves a block, the key tiles taken in turn by its two halves
+      block = dim3(512);
+      if (gh == 4) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 4, TK, 2>), grid, block, 0, stream, p);
+      else if (gh == 2) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 2, TK, 2>), grid, block, 0, stream, p);
+      else hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 1, TK, 2>), grid, block, 0, stream, p);
+      return launch_status();
+    }
+  }
+  if (gh == 4) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 4, TK, 1>), grid, block, 0, stream, p);
+  else if (gh == 2) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 2, TK, 1>), grid, block, 0, stream, p);
+  else hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 1, TK, 1>), grid, block, 0, stream, p);
   return launch_status();
 }
 
@@ -1215,10 +1309,10 @@ ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const
   if (tiled) {   // tiles of atom_attention_prefill_tile_rows() tokens for the kernel with shared key tiles
     if (!atom_attention_prefill_tile_rows(d, page_size, hq / hkv)) return ATOM_UNSUPPORTED;
     switch (d) {
-      case 64: return launch_prefill_tiled<64>(p, num_tiles, rows_per_tile, stream);
-      case 128: return launch_prefill_tiled<128>(p, num_tiles, rows_per_tile, stream);
-      case 192: return launch_prefill_tiled<192>(p, num_tiles, rows_per_tile, stream);
-      case 256: return launch_prefill_tiled<256>(p, num_tiles, rows_per_tile, stream);
+      case 64: return launch_prefill_tiled<64>(p, num_tiles, rows_per_tile, tiled > 1, stream);
+      case 128: return launch_prefill_tiled<128>(p, num_tiles, rows_per_tile, tiled > 1, stream);
+      case 192: return launch_prefill_tiled<192>(p, num_tiles, rows_per_tile, tiled > 1, stream);
+      case 256: return launch_prefill_tiled<256>(p, num_tiles, rows_per_tile, tiled > 1, stream);
       default: return ATOM_UNSUPPORTED;
     }
   }

@@ -166,6 +166,9 @@ class HipKernels:
         self.rows_waves = 0     # 4 or 8 forces the waves a block of that kernel (0: its own choice)
         self.use_mfma_attention = True
         self.use_tiled_prefill = True
+        # Its blocks have eight waves whose halves take the key tiles in turn (D <= 128): True, False, or None for the
+        # choice by the size of the launch (see _prefill_in_halves)
+        self.prefill_key_halves = None
         self.use_fused_decode = True    # decode-only steps of few rows: norm, rotation and cache write inside attention
         self._ws: dict[str, torch.Tensor] = {}
         self._zeroed: dict[str, torch.Tensor] = {}   # workspaces that every kernel leaves all zero
@@ -470,7 +473,8 @@ class HipKernels:
                 # long portions: the kernel whose waves share key tiles through LDS
                 want = self.lib.atom_attention_prefill_tile_rows(d, page_size, hq // hkv)
                 if want and want in meta.tiles_by_rows:
-                    tiles, rows, tiled = meta.tiles_by_rows[want], want, 1
+                    tiles, rows = meta.tiles_by_rows[want], want
+                    tiled = 2 if self._prefill_in_halves(tiles.shape[0] * hq * 32 // (4 * want), meta) else 1
             self._check("prefill tiles", tiles, torch.int32, (None, 2))
             if not tiled and rows not in (16, 32):
                 raise KernelError("attention: tiles hold 16 or 32 rows")
@@ -492,6 +496,21 @@ class HipKernels:
                 _ptr(bt), bt.shape[1], meta.num_prefill, seqs, hq, hkv, d, page_size, ctypes.c_float(scale),
                 int(window or 0), parts, _ptr(ws_o), _ptr(ws_ml), self._stream()))
         return out
+
+    def _prefill_in_halves(self, blocks: int, meta) -> bool:
+        """Whether the prefill kernel with shared key tiles runs blocks of eight waves (one a CU, the key tiles taken
+        in turn by the block's halves) rather than of four (two a CU, each on its own).  Measured on an MI355X with
+        32 / 8 heads of 128: two blocks of four waves keep each other's SIMDs busy as long as both run, so they win
+        when a CU has a queue of them (8,192 fresh tokens: 640 against 690 us) or when all blocks are about as long
+        (2,048 tokens behind 8,192 cached: 355 against 390 us); a block of eight waves does not depend on a
+        neighbour, and wins when there is none (a portion of 512 tokens behind 3,072 cached, 128 blocks: 74 against
+        99 us) or when the long blocks of a fresh prompt outlive their short neighbours (2,048 tokens: 64 against
+        72 us)."""
+        if self.prefill_key_halves is not None:
+            return bool(self.prefill_key_halves)
+        if blocks <= self.num_cus:
+            return True
+        return blocks <= 2 * self.num_cus and 2 * meta.max_context_len < 3 * meta.max_q_len
 
     def fused_decode_attention(self, qkv, k_cache, v_cache, out, meta: AttentionMeta, scale: float, window, q_weight,
                                k_weight, cos, sin, slots, num_heads: int, num_kv_heads: int, head_dim: int,

@@ -298,39 +298,47 @@ def test_prefill_with_shared_key_tiles(hq, hkv, d, page, window):
     q, kc, vc, meta = _attention_case(torch.bfloat16, hq, hkv, d, page, window, q_lens, ctx_lens, seed=hq + d)
     want = torch.empty_like(q)
     PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, window)
-    outs = {}
-    for tiled in (True, False):
-        ops.use_tiled_prefill = tiled
+    # the kernel with shared tiles in blocks of four waves and of eight (the key tiles taken in turn by the block's
+    # halves; head sizes up to 128), then the kernel whose waves load their own keys
+    for tiled, halves in ((True, False), (True, True), (False, None)):
+        ops.use_tiled_prefill, ops.prefill_key_halves = tiled, halves
         try:
             out = torch.zeros_like(q, device=DEV)
             ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, window)
         finally:
-            ops.use_tiled_prefill = True
+            ops.use_tiled_prefill, ops.prefill_key_halves = True, None
         close(out, want, torch.bfloat16)
-        outs[tiled] = out
-    assert not torch.equal(outs[True], outs[False]) or True   # two kernels; both within a bfloat16 ulp of plain
 
 
-def test_prefill_tiles_find_a_far_key():
-    """One key 1,500 positions back, scaled so that its score stands out: the last row must return its value."""
+@pytest.mark.parametrize("halves,far", [(False, 300), (True, 300), (True, 364)])
+def test_prefill_tiles_find_a_far_key(halves, far):
+    """One key about 1,500 positions back, scaled so that its score stands out: the last row must return its value.
+    With blocks of eight waves the key lies once in a tile of the first half (300 = 4 * 64 + 44) and once in a tile
+    of the second (364 = 5 * 64 + 44), whose result reaches the output through the sum of the halves."""
     hq, hkv, d, page = 8, 2, 128, 16
     q_lens, ctx_lens = [96, 1], [1800, 5]
     q, kc, vc, meta = _attention_case(torch.bfloat16, hq, hkv, d, page, None, q_lens, ctx_lens, seed=9,
-                                      scale_one=(0, 300, 4.0))
+                                      scale_one=(0, far, 4.0))
     out = torch.empty_like(q, device=DEV)
-    gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, None)
+    ops = gpu_ops()
+    ops.prefill_key_halves = halves
+    try:
+        ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, None)
+    finally:
+        ops.prefill_key_halves = None
     want = torch.empty_like(q)
     PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, None)
     close(out, want, torch.bfloat16)
     m = meta("cpu")
-    pg, off = int(m.block_tables[0, 300 // page]), 300 % page
+    pg, off = int(m.block_tables[0, far // page]), far % page
     for h in range(hq // hkv - 1, hq, hq // hkv):   # the key was made for the last head of each group
         got, val = out[95, h].float().cpu(), vc[pg, h // (hq // hkv), :, off].float()
         assert float((got - val).abs().max()) < 0.05 * float(val.abs().max()) + 0.05
 
 
+@pytest.mark.parametrize("halves", [False, True])
 @pytest.mark.parametrize("per_tile", [3.0, 11.0])
-def test_prefill_scores_that_climb_from_tile_to_tile(per_tile):
+def test_prefill_scores_that_climb_from_tile_to_tile(per_tile, halves):
     """Every query's scores rise with the key's position, by `per_tile` powers of two from one tile of 64 keys to
     the next: below the step at which the tiled kernel moves a row's running maximum (so that the weights of many
     tiles are taken against an older maximum) and above it (so that it moves with every tile)."""
@@ -348,7 +356,12 @@ def test_prefill_scores_that_climb_from_tile_to_tile(per_tile):
         kf[int(tables[0, key // page]), :, key % page] += per_key * key * u
     kc = kf.to(torch.bfloat16)
     out = torch.empty_like(q, device=DEV)
-    gpu_ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, None)
+    ops = gpu_ops()
+    ops.prefill_key_halves = halves    # with halves the two running maxima differ by a tile's step when they are added
+    try:
+        ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, None)
+    finally:
+        ops.prefill_key_halves = None
     want = torch.empty_like(q)
     PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, None)
     close(out, want, torch.bfloat16)
