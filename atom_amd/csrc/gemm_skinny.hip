@@ -307,14 +307,84 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
     for (int rg = 0; rg < 4; ++rg)
       if (xmine[rg]) xa[4 * slot + rg] = in ? *reinterpret_cast<const bf16x8*>(xrow[rg] + kk) : zero;
   };
+  // The products of a chunk.  The operands of step u + 1 are read from LDS before the products of step u are
+  // issued, and the order is pinned: left to itself the compiler reads each operand right before the product
+  // that takes it and waits for it there.
+  auto multiply = [&](const char* buf) {
+    bf16x8 av[2], bv[2][MT];
+    auto operands = [&](int slot, int u) {
+      av[slot] = *reinterpret_cast<const bf16x8*>(buf + (16 * wave + r16) * kARow + u * 64 + g * 16);
 #pragma unroll
-  for (int slot = 0; slot < kMidAhead; ++slot)
-    if (slot < total) {
-      load_w(slot, slot);
-      load_x(slot, slot);
+      for (int t = 0; t < MT; ++t)
+        bv[slot][t] = *reinterpret_cast<const bf16x8*>(buf + (16 * (waves + t) + r16) * kARow + u * 64 + g * 16);
+    };
+    operands(0, 0);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (u < 3) operands((u + 1) & 1, u + 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u & 1], bv[u & 1][t], acc[t], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
+  };
 
-  for (int base = 0; base < total; base += kMidAhead) {
+  // A range of K that is whole chunks and long enough runs its middle without a branch: every wave brings four
+  // pieces of x a chunk (those beyond the 4 MT that there are bring one of them again, to the same place), and
+  // every chunk's successor exists.  The compiler counts the loads in flight exactly only in straight-line code;
+  // with loads inside branches it waits for every one of them once a trip, which empties the queue that the
+  // loads ahead are there to keep full.
+  int base = 0;
+  if (EXACT && total >= 2 * kMidAhead) {
+    const bf16_t* xrow_all[4];
+    int xat_all[4];
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      const int four = (wave + waves * rg) % (4 * MT);
+      xat_all[rg] = (16 * waves + 4 * four + g) * kARow + r16 * 16;
+      xrow_all[rg] = p.x + (size_t)(m_base + min(4 * four + g, m_rows - 1)) * k + 8 * r16;
+    }
+    auto load_both = [&](int slot, int ci) {
+      const int kk = k_of(ci);
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg)
+        a[4 * slot + rg] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[rg] + kk));
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) xa[4 * slot + rg] = *reinterpret_cast<const bf16x8*>(xrow_all[rg] + kk);
+    };
+    // (in the order of the chunks, pinned: the loop's waits are counted from the order in which the loads went out,
+    // here as in the loop, and the compiler would otherwise send the first chunk's loads last)
+#pragma unroll
+    for (int slot = 0; slot < kMidAhead; ++slot) {
+      load_both(slot, slot);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    for (; base + 2 * kMidAhead <= total; base += kMidAhead) {
+#pragma unroll
+      for (int c = 0; c < kMidAhead; ++c) {
+        const int ci = base + c;
+        char* buf = lds + (ci & 1) * chunk_bytes;
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg)
+          *reinterpret_cast<bf16x8*>(buf + (16 * wave + 4 * rg + g) * kARow + r16 * 16) = a[4 * c + rg];
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) *reinterpret_cast<bf16x8*>(buf + xat_all[rg]) = xa[4 * c + rg];
+        load_both(c, ci + kMidAhead);
+        __syncthreads();
+        multiply(buf);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int slot = 0; slot < kMidAhead; ++slot)
+      if (slot < total) {
+        load_w(slot, slot);
+        load_x(slot, slot);
+      }
+  }
+
+  for (; base < total; base += kMidAhead) {
 #pragma unroll
     for (int c = 0; c < kMidAhead; ++c) {
       const int ci = base + c;
@@ -333,15 +403,7 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
           load_x(c, ci + kMidAhead);
         }
         __syncthreads();
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const bf16x8 av = *reinterpret_cast<const bf16x8*>(buf + (16 * wave + r16) * kARow + u * 64 + g * 16);
-#pragma unroll
-          for (int t = 0; t < MT; ++t) {
-            const bf16x8 bv = *reinterpret_cast<const bf16x8*>(buf + (16 * (waves + t) + r16) * kARow + u * 64 + g * 16);
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc[t], 0, 0, 0);
-          }
-        }
+        multiply(buf);
       }
     }
   }

@@ -135,5 +135,36 @@ def build(force: bool = False) -> str:
     return lib
 
 
+def build_sources(srcs: list[str], lib_name: str, out_dir: str | None = None) -> str:
+    """Compiles HIP sources that are not part of this library (a part that brings kernels of its own) with the
+    library's flags and links them into ``lib_name``; returns its path.  The library lands in ``out_dir``
+    (default: a ``_build`` folder beside the first source, or a per-user temporary folder where that cannot be
+    written) and is rebuilt only when a source is newer.  The sources may include ``common.h`` of this library."""
+    srcs = [os.path.abspath(s) for s in srcs]
+    tag = hashlib.sha1("|".join(srcs).encode()).hexdigest()[:10]
+    candidates = [out_dir] if out_dir else [os.path.join(os.path.dirname(srcs[0]), "_build"),
+                                            os.path.join(tempfile.gettempdir(), f"atom_amd_ext_{os.getuid()}_{tag}")]
+    for folder in candidates:
+        lib = os.path.join(folder, lib_name)
+        if os.path.isfile(lib) and all(os.path.getmtime(s) <= os.path.getmtime(lib) for s in srcs):
+            return lib
+    folder = next((d for d in candidates if _writable(d)), None)
+    if folder is None:
+        raise BuildError(f"no writable build folder among {candidates}")
+    hipcc = _hipcc()
+    _say(f"compiling {len(srcs)} HIP source(s) into {os.path.join(folder, lib_name)}")
+    objs = [os.path.join(folder, os.path.basename(s).rsplit(".", 1)[0] + ".o") for s in srcs]
+    for src, obj in zip(srcs, objs):
+        _compile(hipcc, src, obj)
+    lib = os.path.join(folder, lib_name)
+    tmp = lib + f".tmp{os.getpid()}"
+    res = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs],
+                         stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise BuildError(f"linking {lib} failed:\n{res.stdout}")
+    os.replace(tmp, lib)
+    return lib
+
+
 if __name__ == "__main__":
     print(build(force="--force" in sys.argv))

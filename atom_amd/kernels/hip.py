@@ -171,6 +171,7 @@ class HipKernels:
         self.prefill_key_halves = None
         self.use_fused_decode = True    # decode-only steps of few rows: norm, rotation and cache write inside attention
         self._ws: dict[str, torch.Tensor] = {}
+        self._extensions: dict = {}
         self._zeroed: dict[str, torch.Tensor] = {}   # workspaces that every kernel leaves all zero
         self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
 
@@ -227,6 +228,30 @@ class HipKernels:
         return max(1, min(want, 64, -(-max_context // 64)))
 
     # ------------------------------------------------------------------ helpers
+
+    def load_extension(self, sources: list[str], lib_name: str) -> ctypes.CDLL:
+        """For a part that brings HIP kernels of its own: compiles ``sources`` with this library's flags (once;
+        ``kernels.build.build_sources``) and loads the result.  The part declares its entry points' types on the
+        returned library and calls them with ``pointer(tensor)`` and ``stream()``; ``check`` is the operand test
+        every method here uses."""
+        key = (tuple(sources), lib_name)
+        if key not in self._extensions:
+            try:
+                self._extensions[key] = ctypes.CDLL(_build.build_sources(list(sources), lib_name))
+            except OSError as e:
+                raise KernelError(f"could not load the kernels of {lib_name}: {e}") from e
+        return self._extensions[key]
+
+    def stream(self):
+        """The handle of PyTorch's current stream on this device, as kernels' C entry points take it."""
+        return self._stream()
+
+    @staticmethod
+    def pointer(t: torch.Tensor | None):
+        return _ptr(t)
+
+    def check(self, name: str, t: torch.Tensor, dtype=None, shape=None):
+        return self._check(name, t, dtype, shape)
 
     def _stream(self):
         # the current stream's handle, the short way: these few calls are made hundreds of times a step

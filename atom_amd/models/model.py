@@ -6,12 +6,11 @@ architecture; an architecture is a function from its configuration to a ``ModelS
 from __future__ import annotations
 
 import re
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
 import torch
 
-from ..parts.base import BLOCKS, NORMS, Part, PartChoice
-from ..parts.embedding import LMHead, TokenEmbedding
+from ..parts.base import BLOCKS, EMBEDDINGS, HEADS, NORMS, Part, PartChoice
 
 
 @dataclass(frozen=True)
@@ -31,6 +30,10 @@ class ModelSpec:
     blocks: list[PartChoice]                 # one per layer; kind from the BLOCKS registry
     final_norm: PartChoice
     tie_word_embeddings: bool = False
+    # the embedding and the head, chosen from their registries like every other part; they are built with
+    # vocab_size and hidden_size (the head also with tied_to) beside what the choice names
+    embedding: PartChoice = field(default_factory=lambda: PartChoice("token_embedding"))
+    head: PartChoice = field(default_factory=lambda: PartChoice("lm_head"))
     order: list[LayerRun] | None = None      # default: every layer once, in turn
     max_positions: int = 0
     embedding_prefix: str = "model.embed_tokens"
@@ -52,11 +55,13 @@ class CausalLM(Part):
     def __init__(self, spec: ModelSpec):
         super().__init__("")
         self.spec = spec
-        self.embedding = TokenEmbedding(spec.vocab_size, spec.hidden_size, prefix=spec.embedding_prefix)
+        self.embedding = spec.embedding.build(EMBEDDINGS, vocab_size=spec.vocab_size, hidden_size=spec.hidden_size,
+                                              prefix=spec.embedding_prefix)
         self.blocks = [choice.build(BLOCKS, prefix=spec.layer_prefix.format(i)) for i, choice in enumerate(spec.blocks)]
         self.final_norm = spec.final_norm.build(NORMS, prefix=spec.final_norm_prefix)
-        self.head = LMHead(spec.vocab_size, spec.hidden_size,
-                           tied_to=self.embedding if spec.tie_word_embeddings else None, prefix=spec.head_prefix)
+        self.head = spec.head.build(HEADS, vocab_size=spec.vocab_size, hidden_size=spec.hidden_size,
+                                    tied_to=self.embedding if spec.tie_word_embeddings else None,
+                                    prefix=spec.head_prefix)
         self.order = spec.running_order()
         for i, run in enumerate(self.order):
             if not (0 <= run.layer < len(self.blocks)):

@@ -2,7 +2,7 @@
 
 A *part* owns parameters and computes; it is given every size and constant it needs
 and never learns which model it sits in.  Five kinds are chosen layer by layer from a
-configuration, each through a registry of its own:
+configuration, each through a registry of its own (two more, the embedding and the head, once a model):
 
     mixer              mixes information across positions (attention, or anything with
                        a cache or a per-request state of its own)
@@ -139,6 +139,23 @@ class PositionEncoding(Part):
     """Provides what the mixer's kernels need to encode positions."""
 
 
+class Embedding(Part):
+    """Token ids to the model's first hidden rows.  Built with ``vocab_size``, ``hidden_size`` and whatever
+    else its choice names (a multiplier, say)."""
+
+    def forward(self, ctx, ids: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """Normed hidden rows to float32 logits over the vocabulary.  Built with ``vocab_size``, ``hidden_size``,
+    ``tied_to`` (the model's embedding when the head shares its table, else None) and whatever else its choice
+    names (a cap on the logits, a bias)."""
+
+    def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class Mixer(Part):
     #: True when ``forward`` hands its input to ``ctx.ops.linear`` / ``linear_silu`` as it is and reads nothing of
     #: it but ``shape``, ``dtype`` and ``device``: the norm before the mixer may then be left to that product
@@ -234,6 +251,8 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("head")
 
 
 @dataclass(frozen=True)

@@ -6,10 +6,10 @@ from __future__ import annotations
 
 import torch
 
-from .base import ParamSpec, Part
+from .base import EMBEDDINGS, HEADS, Embedding, Head, ParamSpec
 
 
-class TokenEmbedding(Part):
+class TokenEmbedding(Embedding):
     def __init__(self, vocab_size: int, hidden_size: int, prefix: str = ""):
         super().__init__(prefix)
         self.vocab_size = vocab_size
@@ -23,7 +23,7 @@ class TokenEmbedding(Part):
         return ctx.ops.embedding(self.params["weight"], ids, out)
 
 
-class LMHead(Part):
+class LMHead(Head):
     """``logits = x @ W.T`` in float32 out.  ``tied_to`` names the embedding whose table it shares."""
 
     def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding | None = None, prefix: str = ""):
@@ -43,3 +43,7 @@ class LMHead(Part):
 
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
         return ctx.ops.linear(x, self.weight, None, out_dtype=torch.float32)
+
+
+EMBEDDINGS.register("token_embedding", TokenEmbedding)
+HEADS.register("lm_head", LMHead)

@@ -660,3 +660,101 @@ def test_toy_routed_feed_forward_and_learned_positions(tmp_path):
         FEED_FORWARDS.unregister("routed_toy")
         POSITION_ENCODINGS.unregister("learned_toy")
         unregister_architecture("RoutedToyForCausalLM")
+
+
+# ------------------------------------------------------------------ an embedding and a head with kernels of their own
+
+
+TOY_KERNELS = [__file__.rsplit("/", 1)[0] + "/toy_kernels.hip"]
+
+
+def _toy_lib(ops):
+    """The toy parts' own HIP kernels: compiled with the framework's flags on first use, bound here."""
+    import ctypes
+    lib = ops.load_extension(TOY_KERNELS, "libtoy_kernels.so")
+    lib.toy_scale.restype = lib.toy_softcap.restype = ctypes.c_int
+    return lib
+
+
+class ScaledEmbedding(TokenEmbedding):
+    """The table's rows times a constant (as architectures that scale their embedding by sqrt(hidden) do)."""
+
+    def __init__(self, vocab_size, hidden_size, multiplier: float, prefix=""):
+        super().__init__(vocab_size, hidden_size, prefix)
+        self.multiplier = float(multiplier)
+
+    def forward(self, ctx, ids):
+        import ctypes
+        x = super().forward(ctx, ids)
+        ctx.ops.check("embedded rows", x, (torch.float32, torch.bfloat16), (ids.numel(), self.hidden_size))
+        status = _toy_lib(ctx.ops).toy_scale(ctx.ops.pointer(x), ctypes.c_long(x.numel()), ctypes.c_float(self.multiplier),
+                                             int(x.dtype == torch.bfloat16), ctx.ops.stream())
+        assert status == 0
+        return x
+
+
+class CappedHead(LMHead):
+    """``cap * tanh(logits / cap)``: a soft cap on the logits."""
+
+    def __init__(self, vocab_size, hidden_size, cap: float, tied_to=None, prefix=""):
+        super().__init__(vocab_size, hidden_size, tied_to, prefix)
+        self.cap = float(cap)
+
+    def forward(self, ctx, x):
+        import ctypes
+        logits = super().forward(ctx, x)
+        ctx.ops.check("logits", logits, torch.float32, (x.shape[0], self.vocab_size))
+        status = _toy_lib(ctx.ops).toy_softcap(ctx.ops.pointer(logits), ctypes.c_long(logits.numel()),
+                                               ctypes.c_float(self.cap), ctx.ops.stream())
+        assert status == 0
+        return logits
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding_and_head_with_kernels_of_their_own(dtype, tmp_path):
+    """The embedding and the head come from registries like every other part, and a part may bring HIP code of its
+    own: both toys are defined here, their kernels lie beside this file, and the model that uses them is built,
+    loaded and stepped (decode steps through replayed graphs) without a change to the framework's files."""
+    import dataclasses
+
+    from atom_amd.config.model_config import Qwen3Config
+    from atom_amd.models.qwen3 import qwen3_spec
+    from atom_amd.parts import EMBEDDINGS, HEADS
+    from tiny import TINY_B
+
+    multiplier, cap = 96 ** 0.5, 0.7
+
+    def capped_spec(cfg):
+        return dataclasses.replace(qwen3_spec(cfg), embedding=PartChoice("scaled_embedding", {"multiplier": multiplier}),
+                                   head=PartChoice("capped_head", {"cap": cap}))
+
+    EMBEDDINGS.register("scaled_embedding", ScaledEmbedding)
+    HEADS.register("capped_head", CappedHead)
+    register_architecture("ToyCappedForCausalLM", Qwen3Config, capped_spec)
+    try:
+        raw = dict(TINY_B, architectures=["ToyCappedForCausalLM"])
+        cfg = Qwen3Config.from_dict(raw)
+        folder = write_random_model(str(tmp_path / "capped"), cfg, seed=6, std=0.05, norm_std=0.2)
+        model, _ = load_model(folder, dtype=dtype, device=DEV)
+        assert isinstance(model.embedding, ScaledEmbedding) and isinstance(model.head, CappedHead)
+        core = build_core(model, gpu_ops(), dtype=dtype, device=DEV, page_size=8, num_pages=24, max_num_seqs=2,
+                          graph_sizes=[1, 2])
+        ids = torch.randint(0, cfg.vocab_size, (60,), generator=torch.Generator().manual_seed(3)).tolist()
+        # the plain implementation with the table scaled beforehand and the cap applied afterwards
+        plain_cfg, tensors = pm.load_folder(folder)
+        tensors = dict(tensors)
+        tensors["model.embed_tokens.weight"] = tensors["model.embed_tokens.weight"] * multiplier
+        raw_logits = pm.qwen3_logits(plain_cfg, tensors, ids)
+        want = cap * torch.tanh(raw_logits / cap)
+        assert float(raw_logits.abs().max()) > 1.5 * cap, "the cap must bite for the test to mean something"
+        got = [core.step([StepEntry("r", ids[:40], list(range(40)))]).cpu()]
+        for t in range(40, 60):
+            got.append(core.step([StepEntry("r", [ids[t]], [0])]).cpu())
+        assert core.graphs is not None and core.graphs.replays == 20
+        got = torch.cat(got).double()
+        tol = 1e-4 if dtype == torch.float32 else 4e-2
+        assert float((got - want).abs().max()) <= tol * cap
+    finally:
+        EMBEDDINGS.unregister("scaled_embedding")
+        HEADS.unregister("capped_head")
+        unregister_architecture("ToyCappedForCausalLM")
