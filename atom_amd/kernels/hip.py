@@ -153,7 +153,7 @@ class HipKernels:
                    "atom_attention_mfma_supports", "atom_attention_decode", "atom_attention_prefill",
                    "atom_attention_prefill_tile_rows", "atom_attention_decode_fused",
                    "atom_attention_decode_fused_supports", "atom_gemm_rows", "atom_gemm_rows_parts",
-                   "atom_gemm_rows_supports"):
+                   "atom_gemm_rows_supports", "atom_gemm_tile", "atom_gemm_tile_splits", "atom_gemm_tile_supports"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -163,6 +163,11 @@ class HipKernels:
         # up to 8 bfloat16 rows: the product with the norm before it and the residual sum after it folded in
         self.use_rows_gemm = True
         self.split_library_products = True
+        # 65 to 256 bfloat16 rows, products no wider than 8,192 columns: the kernel whose grid of tiles and K slices
+        # is cut to the chip's CUs (the BLAS library's large tiles leave most of the chip idle there)
+        self.use_tile_gemm = True
+        self.tile_rows = (65, 256)
+        self.tile_max_width = 8192
         self.rows_waves = 0     # 4 or 8 forces the waves a block of that kernel (0: its own choice)
         self.use_mfma_attention = True
         self.use_tiled_prefill = True
@@ -633,6 +638,13 @@ class HipKernels:
                 return slices
         return 1
 
+    def _tile(self, x, weight) -> bool:
+        m, k = x.shape
+        n = weight.shape[0]
+        return bool(self.use_tile_gemm and self.tile_rows[0] <= m <= self.tile_rows[1] and n <= self.tile_max_width
+                    and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                    and self.lib.atom_gemm_tile_supports(m, n, k))
+
     def _skinny(self, x, weight) -> bool:
         m, k = x.shape
         return bool(self.use_skinny_gemm and m <= self.skinny_max_rows and x.dtype == torch.bfloat16
@@ -640,7 +652,8 @@ class HipKernels:
 
     def linear(self, x, weight, bias=None, out_dtype=None, defer: bool = False, few_rows: bool = True):
         """``x @ weight.T (+ bias)``.  bfloat16 operands with at most 64 rows (narrow products: 128) run this
-        library's own weight-streaming kernels; with more rows they go to the BLAS library, as the reference's engine
+        library's own weight-streaming kernels, 65 to 256 rows of products up to 8,192 columns wide its kernel of
+        tiles and K slices cut to the chip; the rest goes to the BLAS library, as the reference's engine
         does for its matrix products; anything with a float32 operand runs this library's float32
         kernel (plain FMA, no reduced-precision mode).  With ``defer`` the result may come back as a
         ``DeferredSum`` for a kernel that adds the slices while it reads them."""
@@ -658,6 +671,20 @@ class HipKernels:
         out_dtype = out_dtype or x.dtype
         if bias is not None:
             self._check("linear bias", bias, torch.float32, (n,))
+        if self._tile(x, weight):
+            splits = self.lib.atom_gemm_tile_splits(m, n, k, self.num_cus)
+            if splits == 1:
+                y = torch.empty((m, n), dtype=out_dtype, device=x.device)
+                self._done("gemm_tile", self.lib.atom_gemm_tile(
+                    _ptr(x), _ptr(weight), _ptr(bias), _ptr(y), None, m, n, k, 1, int(out_dtype == torch.float32),
+                    self._stream()))
+                return y
+            partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+            self._done("gemm_tile", self.lib.atom_gemm_tile(
+                _ptr(x), _ptr(weight), None, None, _ptr(partial), m, n, k, splits, 0, self._stream()))
+            result = DeferredSum(partial, bias, out_dtype)
+            # a product that widens is read next by the rotation kernel, which wants a tensor for this many rows
+            return result if defer and n <= k else self.materialize(result)
         if m and self._skinny(x, weight):
             splits = self.lib.atom_gemm_skinny_splits(m, n, k, 0)
             if splits == 1:

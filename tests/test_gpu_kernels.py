@@ -586,8 +586,10 @@ def all_rows():
     ops = gpu_ops()
     before = ops.skinny_max_rows
     ops.skinny_max_rows = 128
+    ops.use_tile_gemm = False      # (which would take the products of 65 rows and more first)
     yield ops
     ops.skinny_max_rows = before
+    ops.use_tile_gemm = True
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 311, 136), (8, 4096, 4096), (16, 517, 200), (17, 1000, 520), (33, 96, 2056),
@@ -621,6 +623,58 @@ def test_skinny_gemm(m, n, k, out_dtype, all_rows):
     if m > 9:   # more than 8 rows: another kernel, whose cut of K does not depend on the row count
         fewer = ops.linear(x[m - 9:].to(DEV).contiguous(), w.to(DEV), b.to(DEV), out_dtype=out_dtype)
         assert torch.equal(fewer[8], y[m - 1])
+
+
+@pytest.mark.parametrize("m,n,k", [(65, 4096, 4096), (96, 2560, 9728), (128, 6144, 2560), (200, 130, 12288),
+                                   (256, 5120, 5120), (129, 517, 1024), (255, 4096, 12288), (70, 7, 64),
+                                   (100, 1031, 192), (256, 8192, 576)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_tile_gemm(m, n, k, out_dtype):
+    """65 to 256 rows: the kernel of tiles and K slices cut to the chip, at the widths of the 4B, 8B and 32B shapes
+    and at sizes that are no multiple of anything: against the float64 product, whole or left as a sum of slices."""
+    from atom_amd.kernels.hip import DeferredSum
+
+    ops = gpu_ops()
+    x = rnd((m, k), torch.bfloat16, 60, 1.0)
+    w = rnd((n, k), torch.bfloat16, 61, 0.05)
+    b = rnd((n,), torch.float32, 62, 0.5)
+    assert ops._tile(x.to(DEV), w.to(DEV)), "this product must take the tile kernel"
+    want = x.double() @ w.double().T + b.double()
+    ops.allow_library_gemm = False
+    try:
+        y = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), out_dtype=out_dtype)
+        lazy = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), out_dtype=out_dtype, defer=True)
+    finally:
+        ops.allow_library_gemm = True
+    assert y.dtype == out_dtype
+    close(y, want, torch.bfloat16, scale=float(want.abs().max()))
+    if out_dtype == torch.float32:
+        assert float((y.cpu().double() - want).abs().max()) <= 1e-4 * float(want.abs().max())
+    splits = ops.lib.atom_gemm_tile_splits(m, n, k, ops.num_cus)
+    if splits > 1 and n <= k:    # a sum of slices for the norm behind it to add
+        assert isinstance(lazy, DeferredSum) and lazy.splits == splits
+        total = lazy.partial.double().sum(0).cpu() + b.double()
+        assert float((total - want).abs().max()) <= 1e-4 * float(want.abs().max())
+        assert torch.equal(ops.materialize(lazy), y)
+    else:
+        assert torch.equal(lazy, y)
+    # a row's result does not depend on how many rows stand beside it, as long as the tile kernel runs (the
+    # slices of K depend on the number of tiles, so across a tile's edge only within rounding)
+    fewer = ops.linear(x[m - 65:].to(DEV).contiguous(), w.to(DEV), b.to(DEV), out_dtype=out_dtype)
+    close(fewer[64], y[m - 1].double(), torch.bfloat16, scale=float(want.abs().max()))
+
+
+def test_tile_gemm_plan():
+    """The slices of K: the most that keep tiles x slices within the CUs, whole stages, eight of them at least."""
+    lib = gpu_ops().lib
+    assert lib.atom_gemm_tile_splits(256, 4096, 4096, 256) == 4       # 64 tiles
+    assert lib.atom_gemm_tile_splits(256, 6144, 4096, 256) == 2       # 96 tiles
+    assert lib.atom_gemm_tile_splits(96, 4096, 12288, 256) == 8       # 32 tiles
+    assert lib.atom_gemm_tile_splits(128, 2560, 9728, 256) == 8       # 20 tiles
+    assert lib.atom_gemm_tile_splits(128, 2560, 9728 - 64, 256) == 1  # 151 stages: an odd number
+    assert lib.atom_gemm_tile_splits(256, 8192, 576, 256) == 1        # a slice would be shorter than eight stages
+    assert lib.atom_gemm_tile_splits(256, 24576, 4096, 256) == 1      # 384 tiles fill the chip as they are
+    assert lib.atom_gemm_tile_splits(100, 640, 1032, 256) == 0 and not lib.atom_gemm_tile_supports(100, 640, 1032)
 
 
 def test_skinny_gemm_is_what_runs():
