@@ -32,6 +32,7 @@
 #include "linear_static.h"
 
 #include <mutex>
+#include <type_traits>
 
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -330,17 +331,20 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
     }
   };
 
-  // A range of K that is whole chunks and long enough runs its middle without a branch: every wave brings four
-  // pieces of x a chunk (those beyond the 4 MT that there are bring one of them again, to the same place), and
-  // every chunk's successor exists.  The compiler counts the loads in flight exactly only in straight-line code;
-  // with loads inside branches it waits for every one of them once a trip, which empties the queue that the
-  // loads ahead are there to keep full.
+  // A range of K that is whole chunks and long enough runs its middle without a branch: every wave brings the same
+  // number of pieces of x a chunk, XN = ceil(4 MT / waves) (a wave whose piece lies beyond the 4 MT that there are
+  // brings one of them again, to the same place), and every chunk's successor exists.  The compiler counts the
+  // loads in flight exactly only in straight-line code; with loads inside branches it waits for every one of them
+  // once a trip, which empties the queue that the loads ahead are there to keep full.  XN is a constant of the
+  // loop, so the loop is there once for each value that this MT can meet.
   int base = 0;
-  if (EXACT && total >= 2 * kMidAhead) {
-    const bf16_t* xrow_all[4];
-    int xat_all[4];
+  const int x_each = (4 * MT + waves - 1) / waves;
+  auto steady = [&](auto xn) {
+    constexpr int XN = decltype(xn)::value;
+    const bf16_t* xrow_all[XN];
+    int xat_all[XN];
 #pragma unroll
-    for (int rg = 0; rg < 4; ++rg) {
+    for (int rg = 0; rg < XN; ++rg) {
       const int four = (wave + waves * rg) % (4 * MT);
       xat_all[rg] = (16 * waves + 4 * four + g) * kARow + r16 * 16;
       xrow_all[rg] = p.x + (size_t)(m_base + min(4 * four + g, m_rows - 1)) * k + 8 * r16;
@@ -351,7 +355,7 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
       for (int rg = 0; rg < 4; ++rg)
         a[4 * slot + rg] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[rg] + kk));
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) xa[4 * slot + rg] = *reinterpret_cast<const bf16x8*>(xrow_all[rg] + kk);
+      for (int rg = 0; rg < XN; ++rg) xa[4 * slot + rg] = *reinterpret_cast<const bf16x8*>(xrow_all[rg] + kk);
     };
     // (in the order of the chunks, pinned: the loop's waits are counted from the order in which the loads went out,
     // here as in the loop, and the compiler would otherwise send the first chunk's loads last)
@@ -369,13 +373,25 @@ __global__ void __launch_bounds__(512) gemm_mid_kernel(SkinnyParams p) {
         for (int rg = 0; rg < 4; ++rg)
           *reinterpret_cast<bf16x8*>(buf + (16 * wave + 4 * rg + g) * kARow + r16 * 16) = a[4 * c + rg];
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) *reinterpret_cast<bf16x8*>(buf + xat_all[rg]) = xa[4 * c + rg];
+        for (int rg = 0; rg < XN; ++rg) *reinterpret_cast<bf16x8*>(buf + xat_all[rg]) = xa[4 * c + rg];
         load_both(c, ci + kMidAhead);
         __syncthreads();
         multiply(buf);
       }
     }
-  } else {
+  };
+  constexpr int XN_MIN = (4 * MT + 7) / 8;   // with eight waves, the most a block has
+  bool done = false;
+  if (EXACT && total >= 2 * kMidAhead) {
+    if (x_each == XN_MIN) { steady(std::integral_constant<int, XN_MIN>{}); done = true; }
+    if constexpr (MT >= XN_MIN + 1) {
+      if (x_each == XN_MIN + 1) { steady(std::integral_constant<int, XN_MIN + 1>{}); done = true; }
+    }
+    if constexpr (MT >= XN_MIN + 2) {
+      if (x_each == XN_MIN + 2) { steady(std::integral_constant<int, XN_MIN + 2>{}); done = true; }
+    }
+  }
+  if (!done) {
 #pragma unroll
     for (int slot = 0; slot < kMidAhead; ++slot)
       if (slot < total) {
