@@ -368,6 +368,102 @@ def run_long_context(args, contexts=(16384, 32768), batch: int = 8, prefill_toke
     return out
 
 
+def graph_time(fn, variants, reps: int = 3) -> float:
+    """Microseconds a call of ``fn(v)`` takes, from a HIP graph that calls it once for every v in ``variants``
+    (different weights, so that no call finds its operands in a cache), replayed ``reps`` times."""
+    import torch
+
+    stream, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        for v in variants[:2]:
+            fn(v)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            for v in variants:
+                fn(v)
+    graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * len(variants))
+
+
+def run_products(args) -> dict:
+    """The four matrix products of a layer of the chosen shape, alone, at the given numbers of rows: the engine's
+    ``linear`` (whatever kernel it picks, a product left as a sum of slices counted as it is) beside the BLAS
+    library's.  No model is built."""
+    import torch
+    from atom_amd.kernels.hip import HipKernels
+
+    name, raw, _ = SHAPES[args.shape or "8b"]
+    h, d = raw["hidden_size"], raw["head_dim"]
+    hq, hkv, inter = raw["num_attention_heads"], raw["num_key_value_heads"], raw["intermediate_size"]
+    products = [("qkv", (hq + 2 * hkv) * d, h), ("o", h, hq * d), ("gate_up", 2 * inter, h), ("down", h, inter)]
+    ops = HipKernels("cuda:0")
+    rows = [int(v) for v in args.products.split(",")]
+    table = {}
+    for label, n, k in products:
+        copies = max(2, int(2e9 // (n * k * 2)))
+        ws = [torch.randn(n, k, device="cuda:0", dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+        for m in rows:
+            x = torch.randn(m, k, device="cuda:0", dtype=torch.bfloat16)
+            ours = graph_time(lambda w: ops.linear(x, w, None, defer=True), ws)
+            lib = graph_time(lambda w: torch.nn.functional.linear(x, w), ws)
+            flops = 2.0 * m * n * k
+            table[f"{label}_m{m}"] = {"us": round(ours, 1), "library_us": round(lib, 1),
+                                      "tflops": round(flops / ours / 1e6, 1), "weights_gb_s": round(n * k * 2 / ours / 1e3, 1)}
+            print(f"[bench] {label:8s} [{n} x {k}] {m:5d} rows: {ours:7.1f} us ({flops / ours / 1e6:6.1f} TFLOP/s, weights at "
+                  f"{n * k * 2 / ours / 1e6:4.2f} TB/s); BLAS library {lib:7.1f} us", file=sys.stderr, flush=True)
+        del ws
+    return {"metric": f"matrix products of a layer alone ({name} shape, bf16)", "unit": "us", "n_gpus": 1, "dtype": "bf16",
+            "products": table}
+
+
+def run_attention(args) -> dict:
+    """Prefill attention alone: one request brings T tokens behind C cached ones, for every "T,C" pair given."""
+    import torch
+    from atom_amd.kernels.hip import AttentionMeta, HipKernels
+
+    name, raw, _ = SHAPES[args.shape or "8b"]
+    hq, hkv, d, page = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"], 16
+    ops, dev = HipKernels("cuda:0"), "cuda:0"
+    table = {}
+    for pair in args.attention.split(";"):
+        t, cached = (int(v) for v in pair.split(","))
+        ctx = t + cached
+        pages = -(-ctx // page)
+        q = torch.randn(t, hq, d, device=dev, dtype=torch.bfloat16)
+        kc = torch.randn(pages, hkv, page, d, device=dev, dtype=torch.bfloat16)
+        vc = torch.randn(pages, hkv, d, page, device=dev, dtype=torch.bfloat16)
+        out = torch.empty_like(q)
+
+        def tiles_of(rows):
+            starts = sorted(range(0, t, rows), reverse=True)
+            return torch.tensor([(0, r0) for r0 in starts], dtype=torch.int32, device=dev).view(-1, 2)
+
+        short, tall = ops.attention_tile_rows(torch.bfloat16, d, page, hq // hkv, t)
+        meta = AttentionMeta(token_seq=torch.zeros(t, dtype=torch.int32, device=dev),
+                             positions=torch.arange(cached, ctx, dtype=torch.int32, device=dev),
+                             block_tables=torch.arange(pages, dtype=torch.int32, device=dev).view(1, -1),
+                             cu_seqlens_q=torch.tensor([0, t], dtype=torch.int32, device=dev),
+                             context_lens=torch.tensor([ctx], dtype=torch.int32, device=dev), num_seqs=1, num_tokens=t,
+                             max_q_len=t, max_context_len=ctx, page_size=page, num_prefill=1,
+                             prefill_tiles=tiles_of(short), rows_per_tile=short,
+                             tiles_by_rows={tall: tiles_of(tall)} if tall else None)
+        us = graph_time(lambda _: ops.paged_attention(q, kc, vc, out, meta, d ** -0.5), [0] * 8)
+        flops = 4.0 * (t * cached + t * (t + 1) / 2) * d * hq
+        table[f"t{t}_c{cached}"] = {"us": round(us, 1), "tflops": round(flops / us / 1e6, 1),
+                                    "frac": round(flops / us / 1e6 / (MFMA_PEAK["bf16"] / 1e12), 4)}
+        print(f"[bench] prefill attention, {t} tokens behind {cached} cached: {us:8.1f} us, {flops / us / 1e6:6.1f} TFLOP/s",
+              file=sys.stderr, flush=True)
+    return {"metric": f"prefill attention alone ({name} heads, bf16)", "unit": "us", "n_gpus": 1, "dtype": "bf16",
+            "attention": table}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -390,6 +486,11 @@ def main() -> int:
                     help="the prefill and decode points (what --shape 8b runs) on the chosen shape, whatever its own workload")
     ap.add_argument("--single", type=str, default="", metavar="ISL,OSL[;ISL,OSL]",
                     help="one request at a time: TTFT, TPOT and output tok/s, e.g. '18,80;549,256' (the reference's own pairs)")
+    ap.add_argument("--products", type=str, default="", metavar="ROWS[,ROWS]",
+                    help="no model: the four products of a layer of the shape alone at these numbers of rows, the "
+                         "engine's kernels beside the BLAS library's")
+    ap.add_argument("--attention", type=str, default="", metavar="T,C[;T,C]",
+                    help="no model: prefill attention alone, T tokens of one request behind C cached ones")
     ap.add_argument("--budget", type=int, default=None,
                     help="the scheduler's token budget of a step (mixed: 512 + N by default, so that portions stay 512)")
     ap.add_argument("--temperature", type=float, default=0.0, help="of the decode steps' sampling (0: greedy)")
@@ -408,7 +509,10 @@ def main() -> int:
     logging.basicConfig(level=logging.INFO, stream=sys.stderr, format="[bench] %(name)s: %(message)s")
     logging.getLogger("atom_amd").setLevel(logging.INFO if args.shape == "32b" else logging.WARNING)
     # no shape named, nothing else asked for: the headline run and every other shape's workload beside it
-    everything = args.shape is None and not (args.single or args.mixed or args.decode or args.layers)
+    everything = all(getattr(args, k) == ap.get_default(k) for k in vars(args) if k not in ("gpus", "steps", "warmup"))
+    if args.products or args.attention:
+        print(json.dumps(run_products(args) if args.products else run_attention(args)), flush=True)
+        return 0
     args.shape = args.shape or "8b"
     line = run_shape(args)
     if everything:
