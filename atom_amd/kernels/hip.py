@@ -30,6 +30,32 @@ class KernelError(RuntimeError):
     pass
 
 
+@dataclass(frozen=True)
+class ChipFigures:
+    """What was measured on a GPU and decides between two ways of running the same product.  The ways differ in
+    speed and, by rounding, in the last bits of their sums; both are tested against the same reference."""
+
+    stream_bytes_per_us: float     # weights the whole chip streams in a few-rows product, bytes per microsecond
+    cu_bytes_per_us: float         # what a single CU draws at most
+    split_bytes_per_us: float      # the same product with K cut between blocks (more blocks, shorter)
+    add_norm_us: float             # the add-norm kernel that a product cut along K needs beside it
+    library_tile: int              # rows and columns of the BLAS library's large tiles
+    library_slice_k: int           # the least K a slice of a library product keeps ...
+    library_slice_k_many: int      # ... and once there are more than library_many_tiles tiles
+    library_many_tiles: int
+
+
+# by the architecture name the device reports (before its ':' suffixes)
+CHIPS = {
+    # MI355X, 8 rows: a CU draws 28 GB/s at most (22 when all 256 share the chip's 5.6 TB/s); a kernel costs 3.4 us
+    # beside its bytes and the add-norm kernel 5 us.  32B down (320 blocks, 2 on 64 of the CUs): 61.7 us folded
+    # against 48.4 + 5.2 the split way; 32B o: 22.7 against 19.3 + 5.2; 4B down (160 blocks): 14.6 against
+    # 11.2 + 4.7; 8B down (256 blocks): 21.2 against 19.5 + 4.7.
+    "gfx950": ChipFigures(stream_bytes_per_us=5.6e6, cu_bytes_per_us=28e3, split_bytes_per_us=5.5e6, add_norm_us=5.0,
+                          library_tile=256, library_slice_k=2048, library_slice_k_many=4096, library_many_tiles=64),
+}
+
+
 @dataclass
 class AttentionMeta:
     """What attention needs to know about a step's batch, on the device, for one
@@ -178,7 +204,11 @@ class HipKernels:
         self._ws: dict[str, torch.Tensor] = {}
         self._extensions: dict = {}
         self._zeroed: dict[str, torch.Tensor] = {}   # workspaces that every kernel leaves all zero
-        self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
+        props = torch.cuda.get_device_properties(self.device)
+        self.num_cus = props.multi_processor_count
+        arch = str(getattr(props, "gcnArchName", "")).split(":")[0]
+        # the figures of the part these kernels are written for stand in for an unknown one: only speed depends on them
+        self.chip = CHIPS.get(arch, CHIPS["gfx950"])
 
     def workspace(self, name: str, numel: int, dtype=torch.float32) -> torch.Tensor:
         """A scratch tensor that only grows; one per name.  While a HIP graph is being captured the
@@ -336,13 +366,12 @@ class HipKernels:
         """Whether the few-rows product with the residual sum folded in beats the product with K cut between
         blocks followed by the add-norm kernel.  The folded one owns 16 columns and all of K per block, so its
         n / 16 blocks are all the parallelism there is, and it takes as long as its busiest CU needs for its
-        blocks' rows of w.  Measured on an MI355X at 8 rows: a CU draws 28 GB/s at most (22 when all 256 share the
-        chip's 5.6 TB/s), a kernel costs 3.4 us beside that and the add-norm kernel 5 us.  32B down (320 blocks, 2 on
-        64 of the CUs): 61.7 us against 48.4 + 5.2 the split way; 32B o: 22.7 against 19.3 + 5.2; 4B down (160
-        blocks): 14.6 against 11.2 + 4.7; 8B down (256 blocks): 21.2 against 19.5 + 4.7."""
+        blocks' rows of w.  The figures are the chip's (``CHIPS``)."""
+        chip = self.chip
         tiles = -(-n // 16)
-        folded = max(tiles * 32 * k / 5.6e6, -(-tiles // self.num_cus) * 32 * k / 28e3)   # the chip's pace, the busiest CU's
-        split = n * k * 2 / 5.5e6 + 5.0
+        folded = max(tiles * 32 * k / chip.stream_bytes_per_us,                      # the chip's pace,
+                     -(-tiles // self.num_cus) * 32 * k / chip.cu_bytes_per_us)      # the busiest CU's
+        split = n * k * 2 / chip.split_bytes_per_us + chip.add_norm_us
         return folded <= split
 
     def _rows_launch(self, x, weight, bias, mode: int, y=None, res=None, ss_out=None, xg_out=None, g_next=None,
@@ -630,11 +659,12 @@ class HipKernels:
         many rows) are left whole."""
         if not self.split_library_products or n > k:
             return 1
-        tiles = -(-m // 256) * -(-n // 256)
+        chip = self.chip
+        tiles = -(-m // chip.library_tile) * -(-n // chip.library_tile)
         for slices in (4, 2):
             per = k // slices
-            if (k % (slices * 8) == 0 and tiles * slices <= self.num_cus and per >= 2048
-                    and (tiles <= 64 or per >= 4096)):
+            if (k % (slices * 8) == 0 and tiles * slices <= self.num_cus and per >= chip.library_slice_k
+                    and (tiles <= chip.library_many_tiles or per >= chip.library_slice_k_many)):
                 return slices
         return 1
 

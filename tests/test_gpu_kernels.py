@@ -878,6 +878,42 @@ def test_residual_product_with_too_few_tiles_goes_the_split_way():
     close(out, new_res * torch.rsqrt(new_res.pow(2).mean(-1, keepdim=True) + 1e-6) * gamma.double(), torch.bfloat16)
 
 
+@pytest.mark.parametrize("n,k", [(2560, 4096), (2560, 9728), (5120, 8192), (5120, 25600)])
+def test_residual_product_both_ways_at_the_4b_and_32b_widths(n, k):
+    """The o and down products of the 4B and 32B shapes with the residual sum folded in and with K cut between blocks
+    plus the add-norm kernel, whichever of the two the chip's figures choose: both give the reference's residual
+    stream and norm, so the choice changes speed and the last bits only."""
+    from atom_amd.kernels.hip import PendingNorm, PendingProduct
+
+    ops = gpu_ops()
+    m = 6
+    x = rnd((m, k), torch.bfloat16, 80, 1.0)
+    w = rnd((n, k), torch.bfloat16, 81, 0.02)
+    res = rnd((m, n), torch.float32, 82, 2.0)
+    gamma = 1 + rnd((n,), torch.float32, 83, 0.2)
+    new_res = res.double() + x.double() @ w.double().T
+    normed = new_res * torch.rsqrt(new_res.pow(2).mean(-1, keepdim=True) + 1e-6) * gamma.double()
+    chosen = ops._rows_residual_pays(n, k)
+    for folded in (True, False):
+        ops._rows_residual_pays = lambda n_, k_, f=folded: f
+        try:
+            pending = ops.linear(x.to(DEV), w.to(DEV), None, defer=True)
+            assert isinstance(pending, PendingProduct)
+            res_gpu = res.to(DEV)
+            lazy = ops.pending_norm(pending, res_gpu, gamma.to(DEV), 1e-6)
+            if folded:
+                assert isinstance(lazy, PendingNorm)
+                out = ops.materialize(lazy)
+            else:
+                assert lazy is None and pending.split
+                out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+                ops.rmsnorm(pending, gamma.to(DEV), 1e-6, out, residual=res_gpu, mode="add")
+        finally:
+            del ops._rows_residual_pays
+        assert float((res_gpu.cpu().double() - new_res).abs().max()) <= 1e-4 * float(new_res.abs().max()), (folded, chosen)
+        close(out, normed, torch.bfloat16)
+
+
 def test_rows_product_gate_alone_and_odd_widths():
     ops = gpu_ops()
     for m, inter, k in [(1, 200, 136), (8, 12288, 4096), (4, 333, 264), (7, 9, 40)]:
