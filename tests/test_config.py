@@ -149,3 +149,23 @@ def test_cli_renders_prompts_through_the_chat_template(tmp_path):
     text = render_chat(tok, "1+2+3=?")
     assert text == "<|im_start|> user 1+2+3=? <|im_end|> <|im_start|> assistant"
     assert tok.encode(text) == [0, 2, 4, 1, 0, 3]
+
+
+def test_profile_offline_arguments():
+    """The offline profiling command takes the engine's flags and its own four with the reference's defaults
+    (atom/examples/profile_offline.py:19-41), and its prompt is --input-length seeded ids when random."""
+    from types import SimpleNamespace
+
+    from atom_amd.examples import profile_offline as po
+
+    args = po.parser.parse_args(["--model", "m"])
+    assert (args.input_length, args.output_length, args.bs, args.random_input) == (128, 32, 1, False)
+    assert args.torch_profiler_dir is None and po.DEFAULT_TRACE_DIR == "./profiler_traces"
+    args = po.parser.parse_args(["--model", "m", "--input_length", "9", "--bs=4", "--random-input", "--seed", "5"])
+    llm = SimpleNamespace(tokenizer=None, config=SimpleNamespace(model_config=SimpleNamespace(vocab_size=50)))
+    ids = po.make_prompt(llm, args)
+    assert len(ids) == 9 and all(0 <= t < 50 for t in ids) and ids == po.make_prompt(llm, args)
+    args.random_input = False
+    assert po.make_prompt(SimpleNamespace(tokenizer=object(), config=llm.config), args) == po.FIXED_PROMPT
+    with pytest.raises(SystemExit):
+        po.main(["--model", "m", "--bs", "0"])

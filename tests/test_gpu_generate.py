@@ -2,6 +2,7 @@
 long decoding, the first tokens of a sequence, seeded temperature sampling that does not
 depend on the batch, page pressure with preemption, and the command line."""
 
+import os
 import subprocess
 import sys
 
@@ -247,6 +248,22 @@ def test_command_line():
     prompts = [[rng.randrange(256) for _ in range(n)] for n in (5, 17, 33)]
     shown = [eval(m) for m in re.findall(r"Completion: (\[.*?\])", res.stdout)]
     check_greedy("A", "fp32", prompts, [{"token_ids": ids} for ids in shown])
+
+
+def test_profile_offline_command(tmp_path):
+    """The offline profiling command (atom/examples/profile_offline.py:12-117): a warm-up, then --bs equal random
+    prompts between start_profile and stop_profile; the trace holds the steps' spans and this library's kernels."""
+    import json
+    from atom_amd.examples import profile_offline
+    out = str(tmp_path / "traces")
+    outputs = profile_offline.main(["--model", tiny_folder("C"), "--dtype", "bf16", "--block_size", str(PAGE["C"]),
+                                    "--num-kvcache-blocks", "64", "--max-num-seqs", "4", "--input-length", "40",
+                                    "--output-length", "5", "--bs", "3", "--random-input", "--torch-profiler-dir", out])
+    assert len(outputs) == 3 and all(o["num_tokens_input"] == 40 and o["num_tokens_output"] == 5 for o in outputs)
+    with open(os.path.join(out, "trace.json")) as f:
+        names = {e.get("name", "") for e in json.load(f)["traceEvents"]}
+    assert any(n.startswith("prefill[bs=3") for n in names) and any(n.startswith("decode[bs=3") for n in names)
+    assert any("attention" in n and "kernel" in n for n in names), "no kernel of this library in the trace"
 
 
 @pytest.mark.parametrize("which,dtype", [("A", "fp32"), ("B", "fp32"), ("B", "bf16")])
