@@ -57,6 +57,21 @@ struct AttnParams {
 
 __device__ __forceinline__ s16x4 as_s16x4(bf16x4 v) { return __builtin_bit_cast(s16x4, v); }
 
+// The keys of one part of a decode row: the row's visible keys are cut into steps of ``step`` keys (what a wave
+// takes per trip) and the steps are dealt out evenly, the first (steps % parts) parts taking one more.  No part is
+// empty unless there are fewer steps than parts, and no two parts differ by more than one step, whatever the
+// context length: a rule of "ceil(len / parts) rounded up to whole steps" leaves a third of the parts without
+// keys when a part's share is just over two steps.
+struct PartKeys {
+  int begin, end;   // relative to the first visible key; end may lie past the last key
+};
+__device__ inline PartKeys part_keys(int len, int parts, int part, int step) {
+  const int steps = (len + step - 1) / step;
+  const int each = steps / parts, more = steps - each * parts;
+  const int first = part * each + min(part, more);
+  return PartKeys{first * step, (first + each + (part < more ? 1 : 0)) * step};
+}
+
 // Where a key lies: its page's place in the block table and its place in the page.  A power-of-two
 // page size (the usual case) makes these a shift and a mask instead of a division per load.
 // The choice is made once per group of loads (POW2 is a compile-time constant), never per load: a branch
@@ -117,11 +132,9 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
   if (DECODE) {
     int vis = 0;
     if (p.window > 0 && ctx - p.window > 0) vis = (ctx - p.window) & ~15;
-    const int len = ctx - vis;
-    int chunk = (len + p.parts - 1) / p.parts;
-    chunk = (chunk + 15) & ~15;
-    kb = vis + part * chunk;
-    ke = min(ctx, kb + chunk);
+    const PartKeys mine = part_keys(ctx - vis, p.parts, part, 16);
+    kb = vis + mine.begin;
+    ke = min(ctx, vis + mine.end);
   } else {
     kb = 0;
     if (p.window > 0 && pos0 - p.window + 1 > 0) kb = (pos0 - p.window + 1) & ~15;
@@ -382,10 +395,9 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave, (D <= 128 ? 2 : 
 
   int vis0 = 0;
   if (p.window > 0 && ctx - p.window > 0) vis0 = (ctx - p.window) & ~31;
-  int chunk = (ctx - vis0 + p.parts - 1) / p.parts;
-  chunk = (chunk + 31) & ~31;
-  const int kb = vis0 + part * chunk;
-  const int ke = min(ctx, kb + chunk);
+  const PartKeys mine = part_keys(ctx - vis0, p.parts, part, 32);
+  const int kb = vis0 + mine.begin;
+  const int ke = min(ctx, vis0 + mine.end);
 
   f32x4 acc[RT][DT];
   float run_max[RT], run_sum[RT];

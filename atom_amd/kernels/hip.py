@@ -9,6 +9,7 @@ There is no fallback: without a GPU or without the built library, construction f
 from __future__ import annotations
 
 import ctypes
+import math
 from dataclasses import dataclass
 
 import torch
@@ -43,6 +44,7 @@ class ChipFigures:
     library_slice_k: int           # the least K a slice of a library product keeps ...
     library_slice_k_many: int      # ... and once there are more than library_many_tiles tiles
     library_many_tiles: int
+    decode_parts_root: float       # parts of a decode row x sqrt(requests x KV heads) at which attention + merge take least
 
 
 # by the architecture name the device reports (before its ':' suffixes)
@@ -52,7 +54,12 @@ CHIPS = {
     # against 48.4 + 5.2 the split way; 32B o: 22.7 against 19.3 + 5.2; 4B down (160 blocks): 14.6 against
     # 11.2 + 4.7; 8B down (256 blocks): 21.2 against 19.5 + 4.7.
     "gfx950": ChipFigures(stream_bytes_per_us=5.6e6, cu_bytes_per_us=28e3, split_bytes_per_us=5.5e6, add_norm_us=5.0,
-                          library_tile=256, library_slice_k=2048, library_slice_k_many=4096, library_many_tiles=64),
+                          library_tile=256, library_slice_k=2048, library_slice_k_many=4096, library_many_tiles=64,
+                          # decode attention from the QKV product plus the merge, 2 / 4 / 8 requests of 8 KV heads at
+                          # 1,030 to 8,200 keys: least time at 40-64 / 28-48 / 20-28 parts (a part's chain of
+                          # dependent steps shortens with more parts, the merge and the waves' set-up grow); a step
+                          # of 8 requests at 2,100 keys: 3.853 / 3.816 / 3.790 / 3.837 ms with 32 / 28 / 24 / 20 parts
+                          decode_parts_root=192.0),
 }
 
 
@@ -259,7 +266,10 @@ class HipKernels:
     def decode_parts(self, seqs: int, hkv: int, max_context: int) -> int:
         """Over how many waves a decode row's keys are split: enough waves to fill the chip,
         at least 64 keys each."""
-        want = -(-8 * self.num_cus // max(1, seqs * hkv))
+        rows = max(1, seqs * hkv)
+        want = -(-8 * self.num_cus // rows)
+        if want > 8:   # more parts than one block merges itself: the merge kernel's time counts too
+            want = min(want, max(9, round(self.chip.decode_parts_root / math.sqrt(rows))))
         return max(1, min(want, 64, -(-max_context // 64)))
 
     # ------------------------------------------------------------------ helpers
