@@ -3,7 +3,9 @@
 // launches: the RMS norm that precedes a product is applied where the product leaves the matrix cores, and so
 // is the residual sum that follows one.
 //
-// A block owns 16 rows of w (16 output columns) and all of K, which is cut into 8 slices (a function of K
+// A block owns 16 rows of w (16 output columns; 12 or 8 where the caller asks for narrower tiles, so that a
+// width of few tiles spreads over more of the chip's CUs: the matrix cores' tile stays 16 wide and its other
+// columns are dropped) and all of K, which is cut into 8 slices (a function of K
 // alone); its W waves (4 or 8) each walk 8 / W neighbouring slices, a slice's sum in registers of its own.  A wave streams its part of the 16 rows with the whole-cache-line loads of gemm_skinny.hip
 // (non-temporal, 256 contiguous bytes of four rows per load, four quarters of 128 k in flight, each brought
 // into the matrix cores' A operand layout through a wave-private LDS area) and the matching 128 k of x, loaded
@@ -42,6 +44,7 @@ struct RowsParams {
   bf16_t* xg_out;        // residual: [m, n] or null
   const float* g_next;   // residual: [n], the weight of the norm that follows
   int m, n, k, inter, out_f32, mode, ss_parts, kslice, per_wave, tiles;   // kslice: k of a slice; per_wave: slices a wave
+  int cols;              // output columns of a block: 16, 12 or 8 (gate: 8 gate and 8 up rows)
   float eps;
 };
 
@@ -52,9 +55,11 @@ constexpr int kRowsA = 256 + 16;             // LDS bytes of a row of 128 k, 4 b
 constexpr int kRowsAWave = 16 * kRowsA;      // a wave's layout-change area for w
 
 // MR: rows of x that a wave keeps in LDS (the step's row count rounded up to 1, 2, 4 or 8).
-template <int MR>
+// CG: groups of four rows of w that a block owns (4, or 3 or 2 for tiles of 12 or 8 columns).
+template <int MR, int CG>
 // (up to 4 rows: 128 registers, so that a CU holds two blocks of 8 waves)
 __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsParams p) {
+  constexpr int COLS = 4 * CG;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int AREA = kRowsAWave + MR * kRowsA;
   constexpr int XJ = MR > 4 ? 2 : 1;     // 16-byte pieces of x a lane brings per quarter
@@ -76,13 +81,13 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
   // row j (0..15) of the block in w
   auto w_row = [&](int j) -> int {
     if (p.mode == ROWS_GATE) return min(tile * 8 + (j & 7), p.inter - 1) + (j >= 8 ? p.inter : 0);
-    return min(tile * 16 + j, p.n - 1);
+    return min(tile * COLS + j, p.n - 1);
   };
   // a quarter of w: load rg is this lane's 16 bytes of row 4 rg + g at k 8 r16 of the quarter;
   // a quarter of x: piece j is this lane's 16 bytes of row g + 4 j of the batch at the same k
-  const bf16_t* wrow[4];
+  const bf16_t* wrow[CG];
 #pragma unroll
-  for (int rg = 0; rg < 4; ++rg) wrow[rg] = p.w + (size_t)w_row(4 * rg + g) * k + 8 * r16;
+  for (int rg = 0; rg < CG; ++rg) wrow[rg] = p.w + (size_t)w_row(4 * rg + g) * k + 8 * r16;
   const bf16_t* xrow[XJ];
   bool xlive[XJ];
 #pragma unroll
@@ -94,7 +99,7 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
   }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  bf16x8 a[16], xr[4 * XJ];
+  bf16x8 a[4 * CG], xr[4 * XJ];
   auto load_quarter = [&](int q, int slot) {   // quarter q of the wave's range into register slot q % 4
     const int kk = kb + kRowsQuarter * q;
     const bool in = kk + 8 * r16 < ke;
@@ -102,14 +107,15 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
     for (int j = 0; j < XJ; ++j)
       xr[XJ * slot + j] = (in && xlive[j]) ? *reinterpret_cast<const bf16x8*>(xrow[j] + kk) : zero;
 #pragma unroll
-    for (int rg = 0; rg < 4; ++rg)
-      a[4 * slot + rg] = in ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[rg] + kk)) : zero;
+    for (int rg = 0; rg < CG; ++rg)
+      a[CG * slot + rg] = in ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[rg] + kk)) : zero;
   };
   // The norm's factor of every row, from the partial sums of squares in index order: wave v takes rows v and
   // v + waves (there are at least four waves and at most eight rows).  The loads of both rows go out together and
   // ahead of the first quarters of w, so that no wave waits a second time for the cache.
   float* inv_s = reinterpret_cast<float*>(smem + waves * AREA);    // [8], behind the waves' areas
-  float sq[2][4];
+  constexpr int SQ = 8;   // partial sums of squares a lane takes ahead: 512 a row (a width of 6,144 in tiles of 12)
+  float sq[2][SQ];
   if (p.ss) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -117,7 +123,7 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
       const bool live = m < p.m;
       const float* parts = p.ss + (size_t)(p.rows ? p.rows[live ? m : 0] : (live ? m : 0)) * p.ss_parts;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < SQ; ++u) {
         const int i = lane + kWave * u;
         sq[t][u] = (live && i < p.ss_parts) ? parts[i] : 0.f;
       }
@@ -131,10 +137,10 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
     for (int t = 0; t < 2; ++t) {
       const int m = wave + t * waves;
       if (m >= p.m) continue;
-      float sum = (sq[t][0] + sq[t][1]) + (sq[t][2] + sq[t][3]);
-      if (p.ss_parts > 4 * kWave) {
+      float sum = ((sq[t][0] + sq[t][1]) + (sq[t][2] + sq[t][3])) + ((sq[t][4] + sq[t][5]) + (sq[t][6] + sq[t][7]));
+      if (p.ss_parts > SQ * kWave) {
         const float* parts = p.ss + (size_t)(p.rows ? p.rows[m] : m) * p.ss_parts;
-        for (int i = lane + 4 * kWave; i < p.ss_parts; i += kWave) sum += parts[i];
+        for (int i = lane + SQ * kWave; i < p.ss_parts; i += kWave) sum += parts[i];
       }
       sum = wave_sum(sum);
       if (lane == 0) inv_s[m] = rsqrtf(sum / (float)k + p.eps);
@@ -144,6 +150,7 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   float* part = reinterpret_cast<float*>(smem + waves * AREA + 64) + wave * 2 * 16 * 17;   // [2][16 m][16 c + 1]
   const int xread = min(r16, min(MR, p.m) - 1) * kRowsA + 16 * g;   // rows beyond the batch read its last row; not used
+  const int aread = min(r16, COLS - 1) * kRowsA + 16 * g;           // columns beyond the tile read its last; not used
 
   for (int q0 = 0; q0 < quarters; q0 += 4) {
 #pragma unroll
@@ -152,8 +159,8 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
       if (q < quarters) {   // the same in all lanes of the wave
         // the quarter into the operand layouts through the wave's own LDS areas
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg)
-          *reinterpret_cast<bf16x8*>(mine + (4 * rg + g) * kRowsA + r16 * 16) = a[4 * s4 + rg];
+        for (int rg = 0; rg < CG; ++rg)
+          *reinterpret_cast<bf16x8*>(mine + (4 * rg + g) * kRowsA + r16 * 16) = a[CG * s4 + rg];
 #pragma unroll
         for (int j = 0; j < XJ; ++j)
           if (g + 4 * j < MR) *reinterpret_cast<bf16x8*>(xs + (g + 4 * j) * kRowsA + r16 * 16) = xr[XJ * s4 + j];
@@ -167,7 +174,7 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          const bf16x8 av = *reinterpret_cast<const bf16x8*>(mine + r16 * kRowsA + u * 64 + g * 16);
+          const bf16x8 av = *reinterpret_cast<const bf16x8*>(mine + aread + u * 64);
           const bf16x8 bv = *reinterpret_cast<const bf16x8*>(xs + xread + u * 64);
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc, 0, 0, 0);
         }
@@ -211,8 +218,8 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
     }
     return;
   }
-  const int col = tile * 16 + c;
-  const bool has = live && col < p.n;
+  const int col = tile * COLS + c;
+  const bool has = live && c < COLS && col < p.n;
   float v = sum + ((has && p.bias) ? p.bias[col] : 0.f);
   if (p.mode == ROWS_RESIDUAL) {
     float sq = 0.f;
@@ -234,7 +241,8 @@ __global__ void __launch_bounds__(512, (MR > 4 ? 3 : 4)) gemm_rows_kernel(RowsPa
   }
 }
 
-static int rows_tiles(int n, int mode) { return mode == ROWS_GATE ? (n + 7) / 8 : (n + 15) / 16; }
+static int rows_tiles(int n, int mode, int cols) { return mode == ROWS_GATE ? (n + 7) / 8 : (n + cols - 1) / cols; }
+static bool rows_cols_ok(int cols) { return cols == 16 || cols == 12 || cols == 8; }
 
 // Waves a block: enough of them on the chip to keep memory busy, a whole shot of k for each where K allows.
 // Measured on an MI355X: eight waves for the narrow products (a block a CU or little more), four where a CU
@@ -247,8 +255,9 @@ static int rows_waves(int m, int tiles, int k) {
   return waves;
 }
 
-// The number of partial sums of squares a row gets from a product of this width in residual mode.
-ATOM_EXPORT int atom_gemm_rows_parts(int n) { return rows_tiles(n, ROWS_RESIDUAL); }
+// The number of partial sums of squares a row gets from a product of this width in residual mode with
+// tiles of ``cols`` columns (16, 12 or 8; 0 for anything else).
+ATOM_EXPORT int atom_gemm_rows_parts(int n, int cols) { return rows_cols_ok(cols) ? rows_tiles(n, ROWS_RESIDUAL, cols) : 0; }
 
 // 1 if the kernel takes this product.
 ATOM_EXPORT int atom_gemm_rows_supports(int m, int n, int k) {
@@ -256,16 +265,19 @@ ATOM_EXPORT int atom_gemm_rows_supports(int m, int n, int k) {
 }
 
 // mode 0 (plain): y [m, n], bfloat16 or float32 (out_f32).   mode 1 (gate): w is [2 n, k], y [m, n] bfloat16.
-// mode 2 (residual): res [m, n] float32 += product, ss_out [m, atom_gemm_rows_parts(n)], and, with g_next [n],
+// mode 2 (residual): res [m, n] float32 += product, ss_out [m, atom_gemm_rows_parts(n, cols)], and, with g_next [n],
 // xg_out [m, n] = bf16(res * g_next).
+// cols: output columns a block owns in modes 0 and 2: 16, or 12 or 8 for widths whose 16-column tiles would leave
+// CUs without a block or some with one more than others (mode 1 takes 16 only: 8 gate and 8 up rows).
 // Input: x [*, k] bfloat16, row rows[i] of it for row i of the product when rows is given; with ss
 // [*, ss_parts] x is the rows of a float32 stream times a norm's weight, ss the partial sums of squares of those
 // rows, and the product is that of the stream's RMS norm (eps).
 ATOM_EXPORT int atom_gemm_rows(const void* x, const int* rows, const float* ss, int ss_parts, float eps, const void* w,
                                const float* bias, void* y, float* res, float* ss_out, void* xg_out,
-                               const float* g_next, int m, int n, int k, int mode, int out_f32, int waves_override,
-                               hipStream_t stream) {
+                               const float* g_next, int m, int n, int k, int mode, int out_f32, int cols,
+                               int waves_override, hipStream_t stream) {
   if (m < 0 || n <= 0 || k <= 0 || mode < 0 || mode > 2) return ATOM_BAD_SHAPE;
+  if (!rows_cols_ok(cols) || (mode == ROWS_GATE && cols != 16)) return ATOM_UNSUPPORTED;
   if (!atom_gemm_rows_supports(max(m, 1), n, k)) return ATOM_UNSUPPORTED;
   if (m == 0) return ATOM_OK;
   if (!x || !w || (ss && ss_parts < 1)) return ATOM_BAD_SHAPE;
@@ -278,7 +290,8 @@ ATOM_EXPORT int atom_gemm_rows(const void* x, const int* rows, const float* ss, 
   p.m = m; p.k = k; p.out_f32 = out_f32; p.mode = mode; p.ss_parts = ss_parts; p.eps = eps;
   p.n = mode == ROWS_GATE ? 2 * n : n;
   p.inter = mode == ROWS_GATE ? n : 0;
-  p.tiles = rows_tiles(n, mode);
+  p.tiles = rows_tiles(n, mode, cols);
+  p.cols = cols;
   int waves = rows_waves(m, p.tiles, k);
   if (waves_override == 4 || waves_override == 8) waves = waves_override;
   // 8 slices of K (4 where K is shorter than 8 quarters): the same for every number of rows and of waves
@@ -289,13 +302,21 @@ ATOM_EXPORT int atom_gemm_rows(const void* x, const int* rows, const float* ss, 
   p.per_wave = slices / waves;
   const int mr = m <= 1 ? 1 : (m <= 2 ? 2 : (m <= 4 ? 4 : 8));
   const size_t lds = (size_t)waves * (kRowsAWave + mr * kRowsA) + 64 + (size_t)waves * 2 * 16 * 17 * 4;
-#define GO_ROWS(MRV) hipLaunchKernelGGL((gemm_rows_kernel<MRV>), dim3(p.tiles), dim3(64 * waves), lds, stream, p)
-  switch (mr) {
-    case 1: GO_ROWS(1); break;
-    case 2: GO_ROWS(2); break;
-    case 4: GO_ROWS(4); break;
-    default: GO_ROWS(8); break;
+#define GO_ROWS(MRV, CGV) \
+  hipLaunchKernelGGL((gemm_rows_kernel<MRV, CGV>), dim3(p.tiles), dim3(64 * waves), lds, stream, p)
+#define GO_ROWS_COLS(MRV)              \
+  switch (cols) {                      \
+    case 8: GO_ROWS(MRV, 2); break;    \
+    case 12: GO_ROWS(MRV, 3); break;   \
+    default: GO_ROWS(MRV, 4); break;   \
   }
+  switch (mr) {
+    case 1: GO_ROWS_COLS(1); break;
+    case 2: GO_ROWS_COLS(2); break;
+    case 4: GO_ROWS_COLS(4); break;
+    default: GO_ROWS_COLS(8); break;
+  }
+#undef GO_ROWS_COLS
 #undef GO_ROWS
   return launch_status();
 }

@@ -50,9 +50,10 @@ class ChipFigures:
 # by the architecture name the device reports (before its ':' suffixes)
 CHIPS = {
     # MI355X, 8 rows: a CU draws 28 GB/s at most (22 when all 256 share the chip's 5.6 TB/s); a kernel costs 3.4 us
-    # beside its bytes and the add-norm kernel 5 us.  32B down (320 blocks, 2 on 64 of the CUs): 61.7 us folded
-    # against 48.4 + 5.2 the split way; 32B o: 22.7 against 19.3 + 5.2; 4B down (160 blocks): 14.6 against
-    # 11.2 + 4.7; 8B down (256 blocks): 21.2 against 19.5 + 4.7.
+    # beside its bytes and the add-norm kernel 5 us.  With tiles of 16 columns: 32B down (320 blocks, 2 on 64 of
+    # the CUs): 60.0 us folded against 47.2 + 5.2 the split way; 32B o: 22.5 against 19.2 + 5.2; 4B down (160
+    # blocks): 14.6 against 11.2 + 4.7; 8B down (256 blocks): 20.3 against 18.3 + 4.7.  With tiles of 12 columns
+    # (427 and 214 blocks): 32B down 52.0 folded, 32B o 20.2, 4B down 13.5.
     "gfx950": ChipFigures(stream_bytes_per_us=5.6e6, cu_bytes_per_us=28e3, split_bytes_per_us=5.5e6, add_norm_us=5.0,
                           library_tile=256, library_slice_k=2048, library_slice_k_many=4096, library_many_tiles=64,
                           # decode attention from the QKV product plus the merge, 2 / 4 / 8 requests of 8 KV heads at
@@ -201,6 +202,7 @@ class HipKernels:
         self.use_tile_gemm = True
         self.tile_rows = (65, 256)
         self.tile_max_width = 8192
+        self.narrow_row_tiles = True   # tiles of 12 or 8 columns in the few-rows product where they spread better
         self.rows_waves = 0     # 4 or 8 forces the waves a block of that kernel (0: its own choice)
         self.use_mfma_attention = True
         self.use_tiled_prefill = True
@@ -372,15 +374,34 @@ class HipKernels:
                     and (isinstance(x, PendingNorm) or x.dtype == torch.bfloat16)
                     and self.lib.atom_gemm_rows_supports(m, weight.shape[0], k))
 
+    def rows_cols(self, n: int) -> int:
+        """Output columns a block of the few-rows product owns for a width of ``n``: 16, or 12 or 8 where that
+        takes at least a fifth off the columns of the busiest CU (2,560 columns are 160 tiles of 16 for 256 CUs,
+        but 214 of 12; 5,120 and 6,144 are 1.25 and 1.5 tiles of 16 a CU, and 1.67 and 2 of 12).  A block streams
+        its columns' rows of w at what one CU draws, so the busiest CU's columns are the product's time wherever
+        the chip as a whole is not the limit."""
+        if not self.narrow_row_tiles:
+            return 16
+        def busiest(cols: int) -> int:   # columns of the CU with the most blocks
+            tiles = -(-n // cols)
+            return -(-tiles // self.num_cus) * cols
+
+        best = 16
+        for cols in (12, 8):
+            if busiest(cols) * 5 <= busiest(16) * 4 and busiest(cols) < busiest(best):
+                best = cols
+        return best
+
     def _rows_residual_pays(self, n: int, k: int) -> bool:
         """Whether the few-rows product with the residual sum folded in beats the product with K cut between
-        blocks followed by the add-norm kernel.  The folded one owns 16 columns and all of K per block, so its
-        n / 16 blocks are all the parallelism there is, and it takes as long as its busiest CU needs for its
+        blocks followed by the add-norm kernel.  The folded one owns ``rows_cols(n)`` columns and all of K per block, so
+        its blocks are all the parallelism there is, and it takes as long as its busiest CU needs for its
         blocks' rows of w.  The figures are the chip's (``CHIPS``)."""
         chip = self.chip
-        tiles = -(-n // 16)
-        folded = max(tiles * 32 * k / chip.stream_bytes_per_us,                      # the chip's pace,
-                     -(-tiles // self.num_cus) * 32 * k / chip.cu_bytes_per_us)      # the busiest CU's
+        cols = self.rows_cols(n)
+        tiles = -(-n // cols)
+        folded = max(n * 2 * k / chip.stream_bytes_per_us,                                  # the chip's pace,
+                     -(-tiles // self.num_cus) * cols * 2 * k / chip.cu_bytes_per_us)       # the busiest CU's
         split = n * k * 2 / chip.split_bytes_per_us + chip.add_norm_us
         return folded <= split
 
@@ -402,7 +423,7 @@ class HipKernels:
             head = (_ptr(x), None, None, 0, ctypes.c_float(0.0))
         self._done("gemm_rows", self.lib.atom_gemm_rows(
             *head, _ptr(weight), _ptr(bias), _ptr(y), _ptr(res), _ptr(ss_out), _ptr(xg_out), _ptr(g_next), m, n, k,
-            mode, int(out_f32), int(self.rows_waves), self._stream()))
+            mode, int(out_f32), 16 if mode == 1 else self.rows_cols(n), int(self.rows_waves), self._stream()))
 
     def _rows_product(self, x, weight, bias, out_dtype):
         y = torch.empty((x.shape[0], weight.shape[0]), dtype=out_dtype, device=weight.device)
@@ -424,7 +445,8 @@ class HipKernels:
         inner = x.x
         if isinstance(inner, PendingNorm) and inner.r.data_ptr() == residual.data_ptr():
             inner = self.materialize(inner)   # the product may not read the rows it adds to
-        ss = torch.empty((m, self.lib.atom_gemm_rows_parts(n)), dtype=torch.float32, device=residual.device)
+        ss = torch.empty((m, self.lib.atom_gemm_rows_parts(n, self.rows_cols(n))), dtype=torch.float32,
+                         device=residual.device)
         xg = torch.empty((m, n), dtype=torch.bfloat16, device=residual.device)
         self._rows_launch(inner, x.weight, x.bias, 2, res=residual, ss_out=ss, xg_out=xg, g_next=weight)
         return PendingNorm(residual, xg, ss, weight, eps, rows, x.dtype)

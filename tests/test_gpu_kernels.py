@@ -789,12 +789,16 @@ def test_feed_tokens():
 
 @pytest.mark.parametrize("m", [1, 2, 3, 5, 8])
 @pytest.mark.parametrize("n,k", [(311, 136), (4096, 4096), (6144, 2560), (130, 12288), (16, 8), (1031, 520), (5000, 9728)])
-@pytest.mark.parametrize("waves", [0, 4, 8])
-def test_rows_product_plain_gate_and_residual(m, n, k, waves):
+@pytest.mark.parametrize("waves,narrow", [(0, True), (4, True), (8, True), (0, False)])
+def test_rows_product_plain_gate_and_residual(m, n, k, waves, narrow):
+    """(The widths take tiles of 16, 12 and 8 columns a block: 4,096 of 16, 6,144 and 5,000 of 12, the small ones
+    of 8; with ``narrow`` off all take 16.)"""
     from atom_amd.kernels.hip import PendingNorm, PendingProduct
 
     ops = gpu_ops()
     ops.rows_waves = waves
+    ops.narrow_row_tiles = narrow
+    assert [ops.rows_cols(w) for w in (4096, 6144, 5000, 311, 16)] == ([16, 12, 12, 8, 8] if narrow else [16] * 5)
     ops._rows_residual_pays = lambda n, k: True   # the folded residual sum at every size, also where the split way is faster
     try:
         x = rnd((m, k), torch.bfloat16, 50, 1.0)
@@ -848,7 +852,19 @@ def test_rows_product_plain_gate_and_residual(m, n, k, waves):
                 assert torch.equal(y3[0], y2[m - 1]) and torch.equal(y3[1], y2[0])
     finally:
         ops.rows_waves = 0
+        ops.narrow_row_tiles = True
         del ops._rows_residual_pays
+
+
+def test_row_tiles_narrow_where_that_spreads_the_columns():
+    """Tiles of 12 or 8 columns where they take a fifth off the busiest CU's columns (256 CUs): the 4B width (160
+    tiles of 16) and the widths of 1.25 and 1.5 tiles of 16 a CU; not the 8B width, the vocabulary or gate/up."""
+    ops = gpu_ops()
+    assert ops.num_cus == 256
+    assert [ops.rows_cols(n) for n in (2560, 5120, 6144, 3072, 1024)] == [12, 12, 12, 12, 8]
+    assert [ops.rows_cols(n) for n in (4096, 8192, 10240, 151936, 24576, 3584)] == [16] * 6
+    assert ops.lib.atom_gemm_rows_parts(2560, 12) == 214 and ops.lib.atom_gemm_rows_parts(2560, 16) == 160
+    assert ops.lib.atom_gemm_rows_parts(2560, 10) == 0
 
 
 def test_residual_product_with_too_few_tiles_goes_the_split_way():
@@ -859,23 +875,29 @@ def test_residual_product_with_too_few_tiles_goes_the_split_way():
 
     ops = gpu_ops()
     m, n, k = 5, 2560, 26400
-    assert not ops._rows_residual_pays(n, k) and not ops._rows_residual_pays(5120, 25600)
-    assert all(ops._rows_residual_pays(*nk) for nk in [(4096, 12288), (4096, 4096), (2560, 9728), (2560, 4096), (5120, 8192)])
-    x = rnd((m, k), torch.bfloat16, 70, 1.0)
-    w = rnd((n, k), torch.bfloat16, 71, 0.02)
-    want = x.double() @ w.double().T
-    res = rnd((m, n), torch.float32, 72, 2.0)
-    gamma = 1 + rnd((n,), torch.float32, 73, 0.2)
-    pending = ops.linear(x.to(DEV), w.to(DEV), None, defer=True)
-    assert isinstance(pending, PendingProduct)
-    res_gpu = res.to(DEV)
-    assert ops.pending_norm(pending, res_gpu, gamma.to(DEV), 1e-6) is None and pending.split
-    assert isinstance(ops.linear(x.to(DEV), w.to(DEV), None, defer=True, few_rows=False), DeferredSum)
-    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
-    ops.rmsnorm(pending, gamma.to(DEV), 1e-6, out, residual=res_gpu, mode="add")
-    new_res = res.double() + want
-    assert float((res_gpu.cpu().double() - new_res).abs().max()) <= 1e-4 * float(new_res.abs().max())
-    close(out, new_res * torch.rsqrt(new_res.pow(2).mean(-1, keepdim=True) + 1e-6) * gamma.double(), torch.bfloat16)
+    assert all(ops._rows_residual_pays(*nk) for nk in [(4096, 12288), (4096, 4096), (2560, 9728), (2560, 4096), (5120, 8192),
+                                                       (5120, 25600), (n, k)])
+    ops.narrow_row_tiles = False     # with tiles of 16 columns only, these two leave CUs idle for too long
+    try:
+        assert not ops._rows_residual_pays(n, k) and not ops._rows_residual_pays(5120, 25600)
+        assert all(ops._rows_residual_pays(*nk) for nk in [(4096, 12288), (4096, 4096), (2560, 9728), (2560, 4096), (5120, 8192)])
+        x = rnd((m, k), torch.bfloat16, 70, 1.0)
+        w = rnd((n, k), torch.bfloat16, 71, 0.02)
+        want = x.double() @ w.double().T
+        res = rnd((m, n), torch.float32, 72, 2.0)
+        gamma = 1 + rnd((n,), torch.float32, 73, 0.2)
+        pending = ops.linear(x.to(DEV), w.to(DEV), None, defer=True)
+        assert isinstance(pending, PendingProduct)
+        res_gpu = res.to(DEV)
+        assert ops.pending_norm(pending, res_gpu, gamma.to(DEV), 1e-6) is None and pending.split
+        assert isinstance(ops.linear(x.to(DEV), w.to(DEV), None, defer=True, few_rows=False), DeferredSum)
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+        ops.rmsnorm(pending, gamma.to(DEV), 1e-6, out, residual=res_gpu, mode="add")
+        new_res = res.double() + want
+        assert float((res_gpu.cpu().double() - new_res).abs().max()) <= 1e-4 * float(new_res.abs().max())
+        close(out, new_res * torch.rsqrt(new_res.pow(2).mean(-1, keepdim=True) + 1e-6) * gamma.double(), torch.bfloat16)
+    finally:
+        ops.narrow_row_tiles = True
 
 
 @pytest.mark.parametrize("n,k", [(2560, 4096), (2560, 9728), (5120, 8192), (5120, 25600)])
