@@ -821,11 +821,13 @@ static int launch_decode(const AttnParams& p, int seqs, hipStream_t stream) {
 // Needs D % 64 == 0 and page_size % 8 == 0.
 constexpr float kLazyMax = 8.f;
 
-template <int D, int GH, int TK, int KS>
+template <int D, int GH, int TK, int KS, int RT = 2>
 __global__ void __launch_bounds__(256 * KS, (D <= 128 && KS == 1 ? 2 : 1)) attention_prefill_tiled_kernel(AttnParams p) {
   constexpr int KCH = D / 32;
   constexpr int DT = D / 16;
-  constexpr int RT = 2;
+  constexpr int ROWS = 16 * RT;          // query tokens of a wave: 32, or 16 where a launch of 32 would leave CUs idle
+  constexpr int SPLIT = 2 / RT;          // blocks that share an entry of the tile list (which names 32 * 4 / GH tokens)
+  static_assert(RT == 2 || (RT == 1 && KS > 1), "blocks of 16 tokens a wave come with eight waves only");
   constexpr int KB = TK / 16;            // blocks of 16 keys in a tile
   constexpr int KSTR = D + 8;            // LDS row of a key, in elements: rows start 4 banks apart
   constexpr int VSTR = TK + 8;           // LDS row of V^T (one d), in elements: 16-byte aligned, rows 4 banks apart
@@ -859,12 +861,14 @@ __global__ void __launch_bounds__(256 * KS, (D <= 128 && KS == 1 ? 2 : 1)) atten
   // Blocks of eight waves run one a CU and take the items in the order of the list, longest first.
   constexpr bool TWO = D <= 128;
   for (int pass = 0; pass < 2; ++pass) {
-  int tile, ygroup;
+  int tile, ygroup, piece = 0;
   if (KS > 1) {
     if (pass == 1) break;
     const int groups = p.hq / GH;
-    tile = (int)blockIdx.x / groups;
-    ygroup = (int)blockIdx.x - tile * groups;
+    const int unit = (int)blockIdx.x / groups;
+    tile = unit / SPLIT;
+    piece = unit - tile * SPLIT;
+    ygroup = (int)blockIdx.x - unit * groups;
   } else if (TWO) {
     if (pass == 1) break;
     const int total = gridDim.x, half = (total + 1) / 2, groups = p.hq / GH;
@@ -878,19 +882,20 @@ __global__ void __launch_bounds__(256 * KS, (D <= 128 && KS == 1 ? 2 : 1)) atten
   }
   const int seq = p.tiles[2 * tile];
   if (seq < 0) continue;   // an unused entry of a list of fixed length (the same for the whole block)
-  const int row_start = p.tiles[2 * tile + 1];
+  constexpr int TQ = ROWS * (4 / GH);               // tokens of a block
+  const int row_start = p.tiles[2 * tile + 1] + piece * TQ;
   const int head = ygroup * GH + (wave % GH);
   const int kvh = (ygroup * GH) / group;
   const int sub = wave / GH;
   const int ctx = p.ctx_lens[seq];
   const int q_begin = p.cu_q[seq];
   const int q_len = p.cu_q[seq + 1] - q_begin;
-  constexpr int TQ = 32 * (4 / GH);
+  if (row_start >= q_len) continue;                 // the portion ends in the entry's first piece (the whole block)
   const int block_rows = min(TQ, q_len - row_start);
-  const int my_row0 = row_start + 32 * sub;
-  const int nrows = max(0, min(32, q_len - my_row0));
-  const int pos_block0 = ctx - q_len + row_start;   // position of the tile's first token
-  const int pos0 = pos_block0 + 32 * sub;           // of this wave's first token
+  const int my_row0 = row_start + ROWS * sub;
+  const int nrows = max(0, min(ROWS, q_len - my_row0));
+  const int pos_block0 = ctx - q_len + row_start;   // position of the block's first token
+  const int pos0 = pos_block0 + ROWS * sub;         // of this wave's first token
   const int ke = pos_block0 + block_rows;           // one past the last key any row of the block sees
   const int my_ke = pos0 + nrows;
   int kb = 0;
@@ -1181,7 +1186,8 @@ ATOM_EXPORT int atom_attention_prefill_tile_rows(int d, int page_size, int group
 }
 
 template <int D>
-static int launch_prefill_tiled(const AttnParams& p, int num_tiles, int rows_per_tile, bool halves, hipStream_t stream) {
+static int launch_prefill_tiled(const AttnParams& p, int num_tiles, int rows_per_tile, bool halves, bool low,
+                                hipStream_t stream) {
   const int group = p.hq / p.hkv;
   const int gh = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
   if (rows_per_tile != 32 * (4 / gh)) return ATOM_BAD_SHAPE;
@@ -1189,6 +1195,14 @@ static int launch_prefill_tiled(const AttnParams& p, int num_tiles, int rows_per
   if (D <= 128) grid = dim3(num_tiles * (p.hq / gh), 1);
   constexpr int TK = D <= 128 ? 64 : 32;
   if constexpr (D <= 128) {
+    if (halves && low) {   // ... and 16 tokens a wave: two blocks for every entry of the list
+      block = dim3(512);
+      grid = dim3(2 * num_tiles * (p.hq / gh), 1);
+      if (gh == 4) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 4, TK, 2, 1>), grid, block, 0, stream, p);
+      else if (gh == 2) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 2, TK, 2, 1>), grid, block, 0, stream, p);
+      else hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 1, TK, 2, 1>), grid, block, 0, stream, p);
+      return launch_status();
+    }
     if (halves) {   // eight waves a block, the key tiles taken in turn by its two halves
       block = dim3(512);
       if (gh == 4) hipLaunchKernelGGL((attention_prefill_tiled_kernel<D, 4, TK, 2>), grid, block, 0, stream, p);
@@ -1303,7 +1317,9 @@ ATOM_EXPORT int atom_attention_decode_fused(const float* qkv, const float* q_wei
 }
 
 // Prefill: `tiles` lists (request, first row) for every tile of `rows_per_tile` query tokens: 16 or 32 for
-// the kernel in which every wave loads its own keys, atom_attention_prefill_tile_rows() with `tiled`.
+// the kernel in which every wave loads its own keys, atom_attention_prefill_tile_rows() with `tiled` (1: blocks of
+// four waves; 2: of eight waves whose halves take the key tiles in turn; 3: the same with 16 tokens a wave, two
+// blocks for every entry of the list).
 ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
                                        const int* cu_q, const int* ctx_lens, const int* block_tables, int max_blocks,
                                        const int* tiles, int num_tiles, int rows_per_tile, int tiled, int hq, int hkv,
@@ -1321,10 +1337,10 @@ ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const
   if (tiled) {   // tiles of atom_attention_prefill_tile_rows() tokens for the kernel with shared key tiles
     if (!atom_attention_prefill_tile_rows(d, page_size, hq / hkv)) return ATOM_UNSUPPORTED;
     switch (d) {
-      case 64: return launch_prefill_tiled<64>(p, num_tiles, rows_per_tile, tiled > 1, stream);
-      case 128: return launch_prefill_tiled<128>(p, num_tiles, rows_per_tile, tiled > 1, stream);
-      case 192: return launch_prefill_tiled<192>(p, num_tiles, rows_per_tile, tiled > 1, stream);
-      case 256: return launch_prefill_tiled<256>(p, num_tiles, rows_per_tile, tiled > 1, stream);
+      case 64: return launch_prefill_tiled<64>(p, num_tiles, rows_per_tile, tiled > 1, tiled > 2, stream);
+      case 128: return launch_prefill_tiled<128>(p, num_tiles, rows_per_tile, tiled > 1, tiled > 2, stream);
+      case 192: return launch_prefill_tiled<192>(p, num_tiles, rows_per_tile, tiled > 1, tiled > 2, stream);
+      case 256: return launch_prefill_tiled<256>(p, num_tiles, rows_per_tile, tiled > 1, tiled > 2, stream);
       default: return ATOM_UNSUPPORTED;
     }
   }

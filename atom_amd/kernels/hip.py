@@ -209,6 +209,7 @@ class HipKernels:
         # Its blocks have eight waves whose halves take the key tiles in turn (D <= 128): True, False, or None for the
         # choice by the size of the launch (see _prefill_in_halves)
         self.prefill_key_halves = None
+        self.prefill_low_blocks = None   # True / False forces 16 / 32 tokens a wave in the blocks of eight waves
         self.use_fused_decode = True    # decode-only steps of few rows: norm, rotation and cache write inside attention
         self._ws: dict[str, torch.Tensor] = {}
         self._extensions: dict = {}
@@ -565,7 +566,10 @@ class HipKernels:
                 want = self.lib.atom_attention_prefill_tile_rows(d, page_size, hq // hkv)
                 if want and want in meta.tiles_by_rows:
                     tiles, rows = meta.tiles_by_rows[want], want
-                    tiled = 2 if self._prefill_in_halves(tiles.shape[0] * hq * 32 // (4 * want), meta) else 1
+                    blocks = tiles.shape[0] * hq * 32 // (4 * want)
+                    tiled = 2 if self._prefill_in_halves(blocks, meta) else 1
+                    if tiled == 2 and self._prefill_low_blocks(blocks, d):
+                        tiled = 3
             self._check("prefill tiles", tiles, torch.int32, (None, 2))
             if not tiled and rows not in (16, 32):
                 raise KernelError("attention: tiles hold 16 or 32 rows")
@@ -602,6 +606,14 @@ class HipKernels:
         if blocks <= self.num_cus:
             return True
         return blocks <= 2 * self.num_cus and 2 * meta.max_context_len < 3 * meta.max_q_len
+
+    def _prefill_low_blocks(self, blocks: int, head_dim: int) -> bool:
+        """Whether the blocks of eight waves take 16 query tokens a wave instead of 32 (twice the blocks, each with
+        half the products per key tile it stages): when the launch would otherwise leave half of the CUs without a
+        block."""
+        if self.prefill_low_blocks is not None:
+            return bool(self.prefill_low_blocks) and head_dim <= 128
+        return head_dim <= 128 and 2 * blocks <= self.num_cus
 
     def fused_decode_attention(self, qkv, k_cache, v_cache, out, meta: AttentionMeta, scale: float, window, q_weight,
                                k_weight, cos, sin, slots, num_heads: int, num_kv_heads: int, head_dim: int,

@@ -298,20 +298,22 @@ def test_prefill_with_shared_key_tiles(hq, hkv, d, page, window):
     q, kc, vc, meta = _attention_case(torch.bfloat16, hq, hkv, d, page, window, q_lens, ctx_lens, seed=hq + d)
     want = torch.empty_like(q)
     PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, window)
-    # the kernel with shared tiles in blocks of four waves and of eight (the key tiles taken in turn by the block's
-    # halves; head sizes up to 128), then the kernel whose waves load their own keys
-    for tiled, halves in ((True, False), (True, True), (False, None)):
-        ops.use_tiled_prefill, ops.prefill_key_halves = tiled, halves
+    # the kernel with shared tiles in blocks of four waves, of eight (the key tiles taken in turn by the block's
+    # halves; head sizes up to 128) and of eight with 16 tokens a wave (two blocks for every listed tile, the second
+    # of which may lie behind a portion's end), then the kernel whose waves load their own keys
+    for tiled, halves, low in ((True, False, False), (True, True, False), (True, True, True), (False, None, None)):
+        ops.use_tiled_prefill, ops.prefill_key_halves, ops.prefill_low_blocks = tiled, halves, low
         try:
             out = torch.zeros_like(q, device=DEV)
             ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, window)
         finally:
-            ops.use_tiled_prefill, ops.prefill_key_halves = True, None
+            ops.use_tiled_prefill, ops.prefill_key_halves, ops.prefill_low_blocks = True, None, None
         close(out, want, torch.bfloat16)
 
 
-@pytest.mark.parametrize("halves,far", [(False, 300), (True, 300), (True, 364)])
-def test_prefill_tiles_find_a_far_key(halves, far):
+@pytest.mark.parametrize("halves,low,far", [(False, False, 300), (True, False, 300), (True, False, 364), (True, True, 300),
+                                            (True, True, 364)])
+def test_prefill_tiles_find_a_far_key(halves, low, far):
     """One key about 1,500 positions back, scaled so that its score stands out: the last row must return its value.
     With blocks of eight waves the key lies once in a tile of the first half (300 = 4 * 64 + 44) and once in a tile
     of the second (364 = 5 * 64 + 44), whose result reaches the output through the sum of the halves."""
@@ -321,11 +323,11 @@ def test_prefill_tiles_find_a_far_key(halves, far):
                                       scale_one=(0, far, 4.0))
     out = torch.empty_like(q, device=DEV)
     ops = gpu_ops()
-    ops.prefill_key_halves = halves
+    ops.prefill_key_halves, ops.prefill_low_blocks = halves, low
     try:
         ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, None)
     finally:
-        ops.prefill_key_halves = None
+        ops.prefill_key_halves = ops.prefill_low_blocks = None
     want = torch.empty_like(q)
     PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, None)
     close(out, want, torch.bfloat16)
@@ -336,9 +338,9 @@ def test_prefill_tiles_find_a_far_key(halves, far):
         assert float((got - val).abs().max()) < 0.05 * float(val.abs().max()) + 0.05
 
 
-@pytest.mark.parametrize("halves", [False, True])
+@pytest.mark.parametrize("halves,low", [(False, False), (True, False), (True, True)])
 @pytest.mark.parametrize("per_tile", [3.0, 11.0])
-def test_prefill_scores_that_climb_from_tile_to_tile(per_tile, halves):
+def test_prefill_scores_that_climb_from_tile_to_tile(per_tile, halves, low):
     """Every query's scores rise with the key's position, by `per_tile` powers of two from one tile of 64 keys to
     the next: below the step at which the tiled kernel moves a row's running maximum (so that the weights of many
     tiles are taken against an older maximum) and above it (so that it moves with every tile)."""
@@ -358,10 +360,11 @@ def test_prefill_scores_that_climb_from_tile_to_tile(per_tile, halves):
     out = torch.empty_like(q, device=DEV)
     ops = gpu_ops()
     ops.prefill_key_halves = halves    # with halves the two running maxima differ by a tile's step when they are added
+    ops.prefill_low_blocks = low
     try:
         ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), out, meta(DEV), d ** -0.5, None)
     finally:
-        ops.prefill_key_halves = None
+        ops.prefill_key_halves = ops.prefill_low_blocks = None
     want = torch.empty_like(q)
     PLAIN.paged_attention(q, kc, vc, want, meta("cpu"), d ** -0.5, None)
     close(out, want, torch.bfloat16)
