@@ -568,7 +568,7 @@ class HipKernels:
                     tiles, rows = meta.tiles_by_rows[want], want
                     blocks = tiles.shape[0] * hq * 32 // (4 * want)
                     tiled = 2 if self._prefill_in_halves(blocks, meta) else 1
-                    if tiled == 2 and self._prefill_low_blocks(blocks, d):
+                    if tiled == 2 and self._prefill_low_blocks(blocks, d, meta):
                         tiled = 3
             self._check("prefill tiles", tiles, torch.int32, (None, 2))
             if not tiled and rows not in (16, 32):
@@ -607,13 +607,17 @@ class HipKernels:
             return True
         return blocks <= 2 * self.num_cus and 2 * meta.max_context_len < 3 * meta.max_q_len
 
-    def _prefill_low_blocks(self, blocks: int, head_dim: int) -> bool:
+    def _prefill_low_blocks(self, blocks: int, head_dim: int, meta) -> bool:
         """Whether the blocks of eight waves take 16 query tokens a wave instead of 32 (twice the blocks, each with
         half the products per key tile it stages): when the launch would otherwise leave half of the CUs without a
-        block."""
+        block (512 tokens behind 3,072 cached: 65 against 78 us), and for fresh prompts of up to a block a CU, whose
+        blocks are mostly short (549 / 768 / 1,024 tokens: 16 / 20 / 29 against 21 / 24 / 30 us; behind 2,048 cached
+        tokens the same launches take 82-90 against 62-68 us, so those keep 32 tokens a wave)."""
         if self.prefill_low_blocks is not None:
             return bool(self.prefill_low_blocks) and head_dim <= 128
-        return head_dim <= 128 and 2 * blocks <= self.num_cus
+        if head_dim > 128:
+            return False
+        return 2 * blocks <= self.num_cus or (blocks <= self.num_cus and 2 * meta.max_context_len < 3 * meta.max_q_len)
 
     def fused_decode_attention(self, qkv, k_cache, v_cache, out, meta: AttentionMeta, scale: float, window, q_weight,
                                k_weight, cos, sin, slots, num_heads: int, num_kv_heads: int, head_dim: int,
