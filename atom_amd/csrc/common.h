@@ -95,6 +95,20 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   return total;
 }
 
+// The CUs of the current device, asked for once per device: what the launch plans count blocks against (256 on
+// the MI355X that their other figures were measured on; also the answer where no device can be asked).
+static inline int device_cus() {
+  static int known[16] = {0};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 16) return 256;
+  if (!known[device]) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
+    known[device] = cus;
+  }
+  return known[device];
+}
+
 static inline int launch_status() {
   return hipGetLastError() == hipSuccess ? ATOM_OK : ATOM_LAUNCH_FAILED;
 }

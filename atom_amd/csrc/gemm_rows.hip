@@ -246,11 +246,12 @@ static bool rows_cols_ok(int cols) { return cols == 16 || cols == 12 || cols == 
 
 // Waves a block: enough of them on the chip to keep memory busy, a whole shot of k for each where K allows.
 // Measured on an MI355X: eight waves for the narrow products (a block a CU or little more), four where a CU
-// holds several blocks anyway, and from five rows on (two pieces of x a lane and quarter) wherever more than
-// one block a CU is there.
+// holds several blocks anyway (four blocks a CU and more), and from five rows on (two pieces of x a lane and
+// quarter) wherever more than one block a CU is there.
 static int rows_waves(int m, int tiles, int k) {
   const int shots = (k + 511) / 512;
-  int waves = (tiles >= 1024 || (m > 4 && tiles > 256)) ? 4 : 8;
+  const int cus = device_cus();
+  int waves = (tiles >= 4 * cus || (m > 4 && tiles > cus)) ? 4 : 8;
   while (waves > 4 && waves > shots) waves >>= 1;
   return waves;
 }

@@ -529,13 +529,14 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, const fl
 
 static int skinny_tiles(int n, int gate) { return gate ? (n + 31) / 32 : (n + kSkinnyRows - 1) / kSkinnyRows; }
 
-// How K is cut between blocks: slices a multiple of 512.  Measured on an MI355X with the Qwen3-8B
-// products: narrow products (under 256 row tiles) run best with about 512 blocks, wide ones (gate/up,
+// How K is cut between blocks: slices a multiple of 512.  Measured on an MI355X (256 CUs) with the Qwen3-8B
+// products: narrow products (fewer row tiles than CUs) run best with about two blocks a CU, wide ones (gate/up,
 // head) with four slices.
 static SkinnyPlan skinny_plan(int m, int tiles, int k) {
   SkinnyPlan plan{};
   const int units = (k + 511) / 512;
-  int s = tiles >= 256 ? 4 : (512 + tiles - 1) / tiles;
+  const int cus = device_cus();
+  int s = tiles >= cus ? 4 : (2 * cus + tiles - 1) / tiles;
   s = max(1, min(s, min(units, 32)));
   const int per = (units + s - 1) / s;           // units of 512 per slice
   plan.kslice = per * 512;
@@ -550,7 +551,7 @@ static SkinnyPlan skinny_plan(int m, int tiles, int k) {
 // Blocks of 5 to 8 waves run one a CU, blocks of 4 waves two.  Very wide products (three rounds of
 // blocks or more whatever the choice) take four waves and K whole: with two blocks a CU one block's
 // start and end overlap another's work.  For the others the number of waves and of K slices (multiples
-// of 1024) is the one with the least work on the busiest CU: rounds of 256 blocks x rows x k a block,
+// of 1024) is the one with the least work on the busiest CU: rounds of a block a CU x rows x k a block,
 // a little more for fewer waves (x is read once per block), for every round (a block's start and end)
 // and for every slice (its partial sums are written and read again).  The choice does not depend on the number of rows of x.
 struct MidPlan {
@@ -560,7 +561,8 @@ struct MidPlan {
 static MidPlan mid_plan(int groups, int k) {
   MidPlan plan{};
   const int units = (k + kMidSlice - 1) / kMidSlice;
-  if ((groups + 7) / 8 > 2 * 256) {
+  const int cus = device_cus();
+  if ((groups + 7) / 8 > 2 * cus) {
     plan.waves = 4;
     plan.tiles = (groups + 3) / 4;
     plan.splits = 1;
@@ -574,8 +576,8 @@ static MidPlan mid_plan(int groups, int k) {
     if (splits != s) continue;
     for (int w = 8; w >= 4; --w) {
       const long tiles = (groups + w - 1) / w;
-      const long rounds = (tiles * splits + 255) / 256;
-      const double cost = (double)rounds * w * per * (1. + 1. / w) + 0.5 * rounds + 0.15 * splits * groups / 256.;
+      const long rounds = (tiles * splits + cus - 1) / cus;
+      const double cost = (double)rounds * w * per * (1. + 1. / w) + 0.5 * rounds + 0.15 * splits * groups / (double)cus;
       if (cost < best - 1e-9) {
         best = cost;
         plan.waves = w;
@@ -601,7 +603,7 @@ ATOM_EXPORT int atom_gemm_skinny_supports(int m, int n, int k) {
   if (m <= 64) return 1;
   if (m > 128) return 0;
   const MidPlan plan = mid_plan(mid_groups(n, 0), k);   // the same groups with SiLU-gate: n is then twice the columns
-  return plan.waves == 4 && plan.tiles * plan.splits <= 256;
+  return plan.waves == 4 && plan.tiles * plan.splits <= device_cus();
 }
 
 // Into how many slices atom_gemm_skinny cuts K for this product (1: it writes y itself).
